@@ -483,6 +483,77 @@ int32_t nvh_qwen3_exchange_buffers(const nvh_qwen3_model* model, int64_t num_tok
 int32_t nvh_qwen3_logits(const nvh_qwen3_model* model, const void* hidden, const int32_t* cu_seqlens_q,
                          const int32_t* need, int64_t num_rows, void* rows_ws, void* logits, nvh_stream_t stream);
 
+/* ==== Operators for designs outside the Qwen3 family (no counterpart in the reference, which serves Qwen3 only) ====
+ * They lift three limits of the entry points above: the residual stream is fp32 (the sum of the sublayers never rounds
+ * to 16 bits), head sizes and the KV page are arguments, and `act_f32` selects the activation type A of projections,
+ * caches and weights: 0 = bf16, 1 = fp32 (a model served in true 32-bit).  Norm parameters are of type A. */
+
+/* x[T, dim] fp32 = table[ids] (rows outside [0, vocab) give zeros); x0 (may be NULL) receives the same rows in type A. */
+int32_t nvh_embedding_stream(const int64_t* ids, const void* table, float* x, void* x0, int64_t x0_stride,
+                             int64_t num_tokens, int64_t dim, int64_t vocab, int32_t act_f32, nvh_stream_t stream);
+/* Residual add with a Dynamic-Tanh norm on either side, one launch per sublayer boundary.  DyT(v) = tanh(alpha v) w + b
+ * (alpha: one element; no mean, no variance).  Per row:
+ *   s = (accumulate ? x : 0) + post(y) + bias;   x <- s;   h <- next(s)
+ * post / next are skipped when their weight is NULL (no h written without next); y NULL: nothing is added (the stream
+ * is only normalised); bias: one row [dim] of type A added to every row. */
+int32_t nvh_residual_dyt(const void* y, int64_t y_stride, const void* post_alpha, const void* post_w, const void* post_b,
+                         const void* bias, float* x, int32_t accumulate, const void* next_alpha, const void* next_w,
+                         const void* next_b, void* h, int64_t h_stride, int64_t rows, int64_t dim, int32_t act_f32,
+                         nvh_stream_t stream);
+/* out[row, 0:dim] = A(x[row]) (the left half of a [stream | first embedding] row that feeds a looped stack's mixing matrix). */
+int32_t nvh_stream_cast(const float* x, void* out, int64_t out_stride, int64_t rows, int64_t dim, int32_t act_f32, nvh_stream_t stream);
+/* y[rows, inter] = gelu_tanh(gate_up[:, :inter]) * gate_up[:, inter:], evaluated in fp32. */
+int32_t nvh_gelu_tanh_mul(const void* gate_up, int64_t row_stride, void* y, int64_t rows, int64_t inter, int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_gather_rows_f32(const float* x, const int32_t* index, float* out, int64_t rows, int64_t dim, nvh_stream_t stream);
+/* out fp32 [rows, vocab] = cap * tanh(logits / cap) (cap <= 0: a plain conversion to fp32). */
+int32_t nvh_logit_softcap(const void* logits, int64_t row_stride, float* out, int64_t rows, int64_t vocab, float cap, int32_t act_f32,
+                          nvh_stream_t stream);
+/* y[M, N] = x[M, K] w[N, K]^T (+ bias[N]) for ANY sizes and alignments (nvh_gemm_bf16_nt wants K % 64 == 0, N % 4 == 0).
+ * in_f32: operands and bias fp32, products and sums in true fp32 (out_f32 must be set); else bf16 operands on the matrix
+ * cores with fp32 accumulation and a bf16 or fp32 result.  The summation order of an element depends on (N, K) only. */
+int32_t nvh_gemm_any_nt(const void* x, int64_t x_row_stride, const void* w, const void* bias, void* y, int64_t y_row_stride,
+                        int64_t M, int64_t N, int64_t K, int32_t in_f32, int32_t out_f32, nvh_stream_t stream);
+
+/* Attention with a norm over the whole projection, partial rotary, rotated values and a per-head output gate.
+ * nvh_attn_rotary_prep reads the fused projection row [q (H dim) | k (G dim) | v (G vdim) | gate (H, when gate_out)] of
+ * every token: RMS norm (eps, weights of the full projection size) over all of q and all of k; the first rot_dims
+ * dimensions of every q / k head are turned by position * qk_freq[pair] with cos and sin scaled by qk_mag (pairs are
+ * (i, i + rot_dims/2), or (2i, 2i+1) when interleaved; the frequency table carries any scaling rule); the value is
+ * turned by its position over all vdim dimensions with v_freq (NULL: stored as it is).  q -> q_out [T, H dim], k and v ->
+ * cache rows slot_mapping[t] (slot < 0 or NULL caches: not stored), sigmoid(gate) -> gate_out fp32 [T, H]. */
+int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_stride, const void* q_norm_weight, const void* k_norm_weight,
+                             float eps, const int64_t* positions, const float* qk_freq, float qk_mag, int64_t rot_dims,
+                             int32_t qk_interleaved, const float* v_freq, int32_t v_interleaved, void* q_out, float* gate_out,
+                             void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t num_tokens,
+                             int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim, int32_t act_f32,
+                             nvh_stream_t stream);
+/* Causal softmax attention of var-len queries (cu_seqlens_q NULL: one per sequence) over the paged caches
+ * [pages, page, G, dim] / [pages, page, G, vdim]; context_lens counts the keys including this step's.  Scores, weights
+ * and sums in fp32.  Epilogue: each head's output is turned back by the query's position (v_freq; NULL: none) and
+ * multiplied by gate[t, h] (NULL: none).  out [T, H vdim] of type A. */
+int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const void* v_cache, const int32_t* cu_seqlens_q,
+                           const int32_t* context_lens, const int32_t* block_tables, int64_t table_stride, int64_t batch,
+                           int64_t total_q, int64_t page, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
+                           float scale, const float* gate, const float* v_freq, int32_t v_interleaved, void* out,
+                           int32_t act_f32, nvh_stream_t stream);
+
+/* Generalized delta rule, state [slots, H, dk, dv] fp32:  S <- diag(w) S - (a u)(u^T S) + k v^T,  o = S^T r.
+ * nvh_delta_prep: out fp32 [T, 3, H dk] = w | u | a u with w = exp(-decay_scale sigmoid(w0 + w2 tanh(lowrank))),
+ * a = sigmoid(a_raw + a_bias), u = k / sqrt(sum_head k^2 + 1e-6).
+ * nvh_delta_scan: sequence b owns state slot slots[b] (< 0: a padded row) and this step's tokens cu_seqlens_q[b] ..
+ * (NULL: row b); it starts from zero when context_lens[b] equals its token count, else from the slot, and leaves the
+ * state there; out fp32 [T, H dv].  dk % 4 == 0, dk <= 256.
+ * nvh_delta_post: y (type A) = o / rms_head(o) * norm_weight * sigmoid(gate) (gate NULL: none). */
+int32_t nvh_delta_prep(const void* k, int64_t k_stride, const void* a_raw, int64_t a_stride, const void* lowrank, int64_t lowrank_stride,
+                       const void* w2, const void* w0, const void* a_bias, float* out, int64_t num_tokens, int64_t heads, int64_t dk,
+                       int64_t rank, float decay_scale, int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_delta_scan(const void* r, int64_t r_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                       const float* wua, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                       const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
+                       int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_delta_post(const float* o, const void* norm_weight, const void* gate, int64_t gate_stride, void* y, int64_t y_stride,
+                       int64_t rows, int64_t heads, int64_t dv, float eps, int32_t act_f32, nvh_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

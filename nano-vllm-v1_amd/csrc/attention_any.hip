@@ -1,0 +1,326 @@
+// Paged causal attention for any head sizes (query/key size `dim`, value size `vdim`, any page size), with the pieces a
+// gated, value-rotating attention needs around it:
+//   nvh_attn_rotary_prep  per token, over the fused projection row [q | k | v | gate]: RMS norm over the WHOLE q and the
+//                         whole k projection (not per head), partial rotary on q and k (frequency table given by the
+//                         caller, so any scaling rule fits), rotation of the value by its own position over all of
+//                         vdim, sigmoid of the per-head gate; q goes to a packed buffer, k and v to their cache slots.
+//   nvh_attn_paged_any    softmax attention of var-len queries over the paged cache, scores / weights in fp32; the
+//                         epilogue turns each head's output back by the query's position and multiplies the gate.
+// Activations and caches are of type A (bf16 or fp32).  Key tiles always start at key 0 of a sequence and every query
+// row keeps its own running maximum and sum, so a query's result does not depend on how the prompt was cut into steps
+// or on what else is in the batch.
+#include "common.h"
+
+namespace {
+
+template <typename A>
+__device__ __forceinline__ float ldf(const A* p, int64_t i) {
+    return (float)p[i];
+}
+
+__device__ __forceinline__ float block_sum_256(float v, float* scratch) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return scratch[0] + scratch[1] + scratch[2] + scratch[3];
+}
+
+// Index of the rotation partner of element i among `n` rotated dimensions, and the pair number.
+__device__ __forceinline__ void pair_of(int i, int n, int interleaved, int& partner, int& pair, bool& first) {
+    if (interleaved) {
+        partner = i ^ 1;
+        pair = i >> 1;
+        first = (i & 1) == 0;
+    } else {
+        const int half = n >> 1;
+        first = i < half;
+        partner = first ? i + half : i - half;
+        pair = first ? i : i - half;
+    }
+}
+
+struct PrepArgs {
+    const void* proj;          // [T, ld] : q (H*dim) | k (G*dim) | v (G*vdim) | gate (H)
+    int64_t ld;
+    const void *q_norm, *k_norm;   // [H*dim], [G*dim]
+    float eps;
+    const int64_t* positions;
+    const float* qk_freq;      // [rot_dims / 2]
+    float qk_mag;
+    int rot_dims, qk_interleaved;
+    const float* v_freq;       // [vdim / 2], or null: values are stored as they are
+    int v_interleaved;
+    void* q_out;               // [T, H*dim]
+    float* gate_out;           // [T, H], or null (no gate columns in proj)
+    void *k_cache, *v_cache;   // [slots, G*dim], [slots, G*vdim]
+    const int32_t* slot_mapping;
+    int H, G, dim, vdim;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
+    __shared__ float red[4];
+    const int64_t t = blockIdx.x;
+    const A* row = (const A*)a.proj + t * a.ld;
+    const int nq = a.H * a.dim, nk = a.G * a.dim, nv = a.G * a.vdim;
+    const A* qr = row;
+    const A* kr = row + nq;
+    const A* vr = kr + nk;
+    float sq = 0.f, sk = 0.f;
+    for (int i = threadIdx.x; i < nq; i += 256) {
+        const float v = ldf(qr, i);
+        sq += v * v;
+    }
+    for (int i = threadIdx.x; i < nk; i += 256) {
+        const float v = ldf(kr, i);
+        sk += v * v;
+    }
+    sq = block_sum_256(sq, red);
+    sk = block_sum_256(sk, red);
+    const float inv_q = 1.0f / sqrtf(sq / (float)nq + a.eps), inv_k = 1.0f / sqrtf(sk / (float)nk + a.eps);
+    const float pos = (float)a.positions[t];
+    const int64_t slot = a.slot_mapping ? a.slot_mapping[t] : -1;
+    // q and k: norm, then rotary on the first rot_dims dimensions of every head
+    for (int which = 0; which < 2; ++which) {
+        const int n = which ? nk : nq;
+        const A* src = which ? kr : qr;
+        const A* wn = (const A*)(which ? a.k_norm : a.q_norm);
+        const float inv = which ? inv_k : inv_q;
+        A* dst = which ? (slot >= 0 && a.k_cache ? (A*)a.k_cache + slot * nk : nullptr) : (A*)a.q_out + t * nq;
+        if (!dst) continue;
+        for (int i = threadIdx.x; i < n; i += 256) {
+            const int d = i % a.dim;
+            float v = ldf(src, i) * inv * ldf(wn, i);
+            if (d < a.rot_dims) {
+                int partner, pair;
+                bool first;
+                pair_of(d, a.rot_dims, a.qk_interleaved, partner, pair, first);
+                const int j = i - d + partner;
+                const float o = ldf(src, j) * inv * ldf(wn, j);
+                const float ang = pos * a.qk_freq[pair];
+                const float c = cosf(ang) * a.qk_mag, s = sinf(ang) * a.qk_mag;
+                v = first ? v * c - o * s : v * c + o * s;
+            }
+            dst[i] = (A)v;
+        }
+    }
+    if (slot >= 0 && a.v_cache) {
+        A* dst = (A*)a.v_cache + slot * nv;
+        for (int i = threadIdx.x; i < nv; i += 256) {
+            float v = ldf(vr, i);
+            if (a.v_freq) {
+                const int d = i % a.vdim;
+                int partner, pair;
+                bool first;
+                pair_of(d, a.vdim, a.v_interleaved, partner, pair, first);
+                const float o = ldf(vr, i - d + partner);
+                const float ang = pos * a.v_freq[pair];
+                const float c = cosf(ang), s = sinf(ang);
+                v = first ? v * c - o * s : v * c + o * s;
+            }
+            dst[i] = (A)v;
+        }
+    }
+    if (a.gate_out)
+        for (int h = threadIdx.x; h < a.H; h += 256) a.gate_out[t * a.H + h] = 1.0f / (1.0f + expf(-ldf(vr + nv, h)));
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int AQ = 16;        // queries per workgroup (one 16-lane row of a wave per query)
+constexpr int AK = 32;        // keys per tile
+constexpr int AVC = 16;       // value columns per lane: vdim <= 16 * AVC
+
+struct AttnArgs {
+    const void* q;             // [T, H*dim]
+    const void *k_cache, *v_cache;
+    const int32_t* cu_seqlens_q;    // [B+1], or null: one query per sequence (row b is sequence b)
+    const int32_t* context_lens;    // [B]: keys of the sequence including this step's tokens
+    const int32_t* block_tables;
+    int64_t table_stride;
+    int batch, page;
+    int H, G, dim, vdim;
+    float scale;
+    const float* gate;         // [T, H] or null
+    const float* v_freq;       // [vdim/2] or null: no turning back
+    int v_interleaved;
+    void* out;                 // [T, H*vdim]
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
+    extern __shared__ float smem[];
+    // which (sequence, query tile) is this workgroup's
+    int seq = -1, q0 = 0, qlen = 0, qbase = 0;
+    {
+        int tile = blockIdx.x;
+        for (int b = 0; b < a.batch; ++b) {
+            const int lo = a.cu_seqlens_q ? a.cu_seqlens_q[b] : b, hi = a.cu_seqlens_q ? a.cu_seqlens_q[b + 1] : b + 1;
+            const int tiles = (hi - lo + AQ - 1) / AQ;
+            if (tile < tiles) {
+                seq = b;
+                q0 = tile * AQ;
+                qlen = hi - lo;
+                qbase = lo;
+                break;
+            }
+            tile -= tiles;
+        }
+    }
+    if (seq < 0) return;                                     // (uniform over the workgroup)
+    const int head = blockIdx.y, kvh = head / (a.H / a.G);
+    const int dim = a.dim, vdim = a.vdim;
+    const int klen = a.context_lens[seq];
+    const int past = klen - qlen;                            // keys before this step's first query
+    const int nq = min(AQ, qlen - q0);
+    const int kd = dim + 1, vd = vdim + 1;
+    float* qs = smem;                                        // [AQ][dim]
+    float* ks = qs + AQ * dim;                               // [AK][dim + 1]
+    float* vs = ks + AK * kd;                                // [AK][vdim + 1]
+    float* ps = vs + AK * vd;                                // [AQ][AK]
+    const int tid = threadIdx.x, qi = tid >> 4, sub = tid & 15;
+    for (int i = tid; i < AQ * dim; i += 256) {
+        const int r = i / dim, d = i - r * dim;
+        qs[i] = r < nq ? ldf((const A*)a.q, (int64_t)(qbase + q0 + r) * a.H * dim + head * dim + d) * a.scale : 0.f;
+    }
+    float acc[AVC];
+#pragma unroll
+    for (int c = 0; c < AVC; ++c) acc[c] = 0.f;
+    float m_run = -INFINITY, l_run = 0.f;
+    const int qpos = past + q0 + qi;                         // this lane's query position (valid for qi < nq)
+    const int last_key = past + q0 + nq - 1;                 // the tile's last query sees keys 0..last_key
+    const int32_t* table = a.block_tables + (int64_t)seq * a.table_stride;
+    for (int k0 = 0; k0 <= last_key; k0 += AK) {
+        __syncthreads();                                     // the previous tile's readers are done
+        for (int i = tid; i < AK * dim; i += 256) {
+            const int r = i / dim, d = i - r * dim, key = k0 + r;
+            float v = 0.f;
+            if (key <= last_key) {
+                const int64_t slot = (int64_t)table[key / a.page] * a.page + key % a.page;
+                v = ldf((const A*)a.k_cache, (slot * a.G + kvh) * dim + d);
+            }
+            ks[r * kd + d] = v;
+        }
+        for (int i = tid; i < AK * vdim; i += 256) {
+            const int r = i / vdim, d = i - r * vdim, key = k0 + r;
+            float v = 0.f;
+            if (key <= last_key) {
+                const int64_t slot = (int64_t)table[key / a.page] * a.page + key % a.page;
+                v = ldf((const A*)a.v_cache, (slot * a.G + kvh) * vdim + d);
+            }
+            vs[r * vd + d] = v;
+        }
+        __syncthreads();
+        // scores of query qi against keys sub and sub + 16 of the tile
+        float s0 = 0.f, s1 = 0.f;
+        const float* qrow = qs + qi * dim;
+        const float *kr0 = ks + sub * kd, *kr1 = ks + (sub + 16) * kd;
+        for (int d = 0; d < dim; ++d) {
+            const float qv = qrow[d];
+            s0 = __builtin_fmaf(qv, kr0[d], s0);
+            s1 = __builtin_fmaf(qv, kr1[d], s1);
+        }
+        const bool ok0 = qi < nq && k0 + sub <= qpos, ok1 = qi < nq && k0 + sub + 16 <= qpos;
+        s0 = ok0 ? s0 : -INFINITY;
+        s1 = ok1 ? s1 : -INFINITY;
+        const float m_new = fmaxf(m_run, row16_max(fmaxf(s0, s1)));
+        // a row that sees nothing yet keeps m = -inf (only rows past nq: every real query sees key 0)
+        const float p0 = ok0 ? expf(s0 - m_new) : 0.f, p1 = ok1 ? expf(s1 - m_new) : 0.f;
+        const float alpha = m_new == -INFINITY ? 1.f : expf(m_run - m_new);
+        l_run = l_run * alpha + row16_sum(p0 + p1);
+        m_run = m_new;
+        ps[qi * AK + sub] = p0;
+        ps[qi * AK + sub + 16] = p1;
+        __syncthreads();
+        const float* prow = ps + qi * AK;
+#pragma unroll
+        for (int c = 0; c < AVC; ++c) {
+            const int col = sub + 16 * c;
+            if (col < vdim) {
+                float s = acc[c] * alpha;
+                for (int r = 0; r < AK; ++r) s = __builtin_fmaf(prow[r], vs[r * vd + col], s);
+                acc[c] = s;
+            }
+        }
+    }
+    // epilogue: normalise, turn back by the query's position, gate
+    __syncthreads();
+    float* os = ks;                                          // [AQ][vdim] (fits: AK >= AQ)
+#pragma unroll
+    for (int c = 0; c < AVC; ++c) {
+        const int col = sub + 16 * c;
+        if (col < vdim) os[qi * vdim + col] = l_run > 0.f ? acc[c] / l_run : 0.f;
+    }
+    __syncthreads();
+    if (qi < nq) {
+        const int64_t tok = qbase + q0 + qi;
+        const float g = a.gate ? a.gate[tok * a.H + head] : 1.0f;
+        const float pos = (float)qpos;
+#pragma unroll
+        for (int c = 0; c < AVC; ++c) {
+            const int col = sub + 16 * c;
+            if (col < vdim) {
+                float v = os[qi * vdim + col];
+                if (a.v_freq) {
+                    int partner, pair;
+                    bool first;
+                    pair_of(col, vdim, a.v_interleaved, partner, pair, first);
+                    const float o = os[qi * vdim + partner];
+                    const float ang = pos * a.v_freq[pair];
+                    const float cs = cosf(ang), sn = sinf(ang);
+                    v = first ? v * cs + o * sn : v * cs - o * sn;        // the rotation by -pos
+                }
+                ((A*)a.out)[(tok * a.H + head) * vdim + col] = (A)(v * g);
+            }
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_stride, const void* q_norm_weight, const void* k_norm_weight,
+                                        float eps, const int64_t* positions, const float* qk_freq, float qk_mag, int64_t rot_dims,
+                                        int32_t qk_interleaved, const float* v_freq, int32_t v_interleaved, void* q_out, float* gate_out,
+                                        void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t num_tokens,
+                                        int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim, int32_t act_f32,
+                                        nvh_stream_t stream) {
+    NVH_REQUIRE(proj && q_norm_weight && k_norm_weight && positions && q_out, NVH_EINVAL, "nvh_attn_rotary_prep: null pointer");
+    NVH_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && dim > 0 && vdim > 0 && num_tokens >= 0, NVH_EINVAL, "nvh_attn_rotary_prep: bad sizes");
+    NVH_REQUIRE(rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0 && (rot_dims == 0 || qk_freq), NVH_EINVAL,
+                "nvh_attn_rotary_prep: rot_dims %ld does not fit dim %ld", (long)rot_dims, (long)dim);
+    NVH_REQUIRE(!v_freq || vdim % 2 == 0, NVH_EINVAL, "nvh_attn_rotary_prep: rotated values need an even vdim");
+    NVH_REQUIRE(proj_row_stride >= (num_q_heads + num_kv_heads) * dim + num_kv_heads * vdim + (gate_out ? num_q_heads : 0), NVH_EINVAL,
+                "nvh_attn_rotary_prep: projection row too short");
+    if (num_tokens == 0) return NVH_OK;
+    PrepArgs a{proj, proj_row_stride, q_norm_weight, k_norm_weight, eps, positions, qk_freq, qk_mag, (int)rot_dims, qk_interleaved,
+               v_freq, v_interleaved, q_out, gate_out, k_cache, v_cache, slot_mapping, (int)num_q_heads, (int)num_kv_heads, (int)dim, (int)vdim};
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) attn_rotary_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(a);
+    else attn_rotary_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(a);
+    NVH_CHECK_LAUNCH("nvh_attn_rotary_prep");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const void* v_cache, const int32_t* cu_seqlens_q,
+                                      const int32_t* context_lens, const int32_t* block_tables, int64_t table_stride, int64_t batch,
+                                      int64_t total_q, int64_t page, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
+                                      float scale, const float* gate, const float* v_freq, int32_t v_interleaved, void* out,
+                                      int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(q && k_cache && v_cache && context_lens && block_tables && out, NVH_EINVAL, "nvh_attn_paged_any: null pointer");
+    NVH_REQUIRE(batch >= 0 && total_q >= 0 && page > 0 && num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0 && dim > 0 && vdim > 0,
+                NVH_EINVAL, "nvh_attn_paged_any: bad sizes");
+    NVH_REQUIRE(vdim <= 16 * AVC, NVH_ENOSYS, "nvh_attn_paged_any: vdim %ld above %d", (long)vdim, 16 * AVC);
+    NVH_REQUIRE(!v_freq || vdim % 2 == 0, NVH_EINVAL, "nvh_attn_paged_any: rotated values need an even vdim");
+    const size_t lds = sizeof(float) * (size_t)(AQ * dim + AK * (dim + 1) + AK * (vdim + 1) + AQ * AK);
+    NVH_REQUIRE(lds <= 64 * 1024, NVH_ENOSYS, "nvh_attn_paged_any: dim %ld + vdim %ld need %zu bytes of LDS", (long)dim, (long)vdim, lds);
+    if (batch == 0 || total_q == 0) return NVH_OK;
+    AttnArgs a{q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, table_stride, (int)batch, (int)page, (int)num_q_heads,
+               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out};
+    // at most ceil(len / AQ) tiles per sequence: total_q / AQ + batch bounds their number (surplus workgroups exit)
+    const dim3 grid((unsigned)(total_q / AQ + batch), (unsigned)num_q_heads);
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) attn_paged_any_kernel<float><<<grid, 256, lds, st>>>(a);
+    else attn_paged_any_kernel<bf16><<<grid, 256, lds, st>>>(a);
+    NVH_CHECK_LAUNCH("nvh_attn_paged_any");
+    return NVH_OK;
+}

@@ -180,6 +180,11 @@ __device__ __forceinline__ void philox(uint32_t (&c)[4], uint32_t k0, uint32_t k
 // (layers/sampler.py:80, clamp_min_(1e-10)).
 __device__ __forceinline__ void nvh_race_scores(const float (&z)[4], float inv_t, int64_t col, int64_t row, uint64_t seed, uint64_t offset,
                                                 float (&sc)[4]) {
+    if (inv_t == 0.f) {                                      // a greedy row (temperature 0): the plain logits race, no noise
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sc[e] = z[e];
+        return;
+    }
     uint32_t c[4] = {(uint32_t)(col >> 2), (uint32_t)row, (uint32_t)offset, (uint32_t)(offset >> 32)};
     philox(c, (uint32_t)seed, (uint32_t)(seed >> 32));
     constexpr float LN2 = 0.6931471805599453f;

@@ -1,0 +1,213 @@
+// Generalized delta rule: a per-head matrix state S [dk, dv] in fp32 that every token updates,
+//   S <- diag(w) S - (a * u) (u^T S) + k v^T     (both terms read the old S),   o = S^T r,
+// with a decay w in (0, 1) and a removal rate a per key channel and u the unit-length key.
+//   nvh_delta_prep   per token and channel, all in fp32: the decay from its low-rank logit
+//                    w = exp(-c * sigmoid(w0 + W2 tanh(l))) (c = e^-1/2 by default), a = sigmoid(a_raw + a_bias),
+//                    u = k / sqrt(sum k^2 + 1e-6); leaves [w | u | a*u] per token.
+//   nvh_delta_scan   walks a sequence's tokens in order from the state its slot holds (or from zero when the sequence
+//                    starts) and leaves the state there.  Columns of S are independent of each other, so the work is
+//                    spread over (sequence, head, column); each column is held by four lanes (rows i mod 4), which
+//                    meet twice per token in a quad sum.  The order of every sum is fixed by the sizes alone: decoding
+//                    token by token, in portions or in one piece gives the same bits.
+//   nvh_delta_post   per head: o / rms(o), times the norm weight and the sigmoid output gate, to the activation type.
+#include "common.h"
+
+namespace {
+
+template <typename A>
+__device__ __forceinline__ float ldf(const A* p, int64_t i) {
+    return (float)p[i];
+}
+__device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
+
+struct DeltaPrepArgs {
+    const void* k;             // [T, ld] rows of H*dk
+    int64_t k_stride;
+    const void* a_raw;         // [T, ld]
+    int64_t a_stride;
+    const void* lowrank;       // [T, ld] rows of `rank` (the first decay projection, before its tanh)
+    int64_t l_stride;
+    const void *w2, *w0, *a_bias;   // [H*dk, rank], [H*dk], [H*dk]
+    float* out;                // [T, 3, H*dk]: w | u | a*u
+    int H, dk, rank;
+    float decay_scale;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepArgs p) {
+    extern __shared__ float tl[];                            // tanh of the low-rank row
+    const int64_t t = blockIdx.x;
+    const int n = p.H * p.dk;
+    for (int r = threadIdx.x; r < p.rank; r += 256) tl[r] = tanhf(ldf((const A*)p.lowrank, t * p.l_stride + r));
+    __syncthreads();
+    float* out = p.out + t * 3 * n;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int h = wave; h < p.H; h += 4) {
+        float ss = 0.f;
+        for (int i = lane; i < p.dk; i += 64) {
+            const float kv = ldf((const A*)p.k, t * p.k_stride + h * p.dk + i);
+            ss += kv * kv;
+        }
+        ss = wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss + 1e-6f);
+        for (int i = lane; i < p.dk; i += 64) {
+            const int c = h * p.dk + i;
+            float z = ldf((const A*)p.w0, c);
+            const A* w2r = (const A*)p.w2 + (int64_t)c * p.rank;
+            for (int r = 0; r < p.rank; ++r) z = __builtin_fmaf(ldf(w2r, r), tl[r], z);
+            const float u = ldf((const A*)p.k, t * p.k_stride + c) * inv;
+            const float a = sigmoidf_(ldf((const A*)p.a_raw, t * p.a_stride + c) + ldf((const A*)p.a_bias, c));
+            out[c] = expf(-p.decay_scale * sigmoidf_(z));
+            out[n + c] = u;
+            out[2 * n + c] = a * u;
+        }
+    }
+}
+
+struct DeltaScanArgs {
+    const void *r, *k, *v;     // [T, stride] rows of H*dk (r, k) and H*dv (v)
+    int64_t r_stride, k_stride, v_stride;
+    const float* wua;          // [T, 3, H*dk]
+    float* state;              // [slots, H, dk, dv]
+    const int32_t* slots;      // [B]
+    const int32_t* cu_seqlens_q;    // [B+1] or null (one token per sequence)
+    const int32_t* context_lens;    // [B]: tokens of the sequence including this step's (a step that holds them all starts from zero)
+    float* out;                // [T, H*dv]
+    int H, dk, dv;
+};
+
+constexpr int DTOK = 8;        // tokens staged per round
+
+template <typename A, int DKQ>
+__global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
+    extern __shared__ float sm[];                            // [DTOK][5 dk + dv]: r | k | w | u | au | v
+    const int seq = blockIdx.x, head = blockIdx.y;
+    const int dk = p.dk, dv = p.dv, dkq = dk >> 2;
+    const int col = blockIdx.z * 64 + (threadIdx.x >> 2), sub = threadIdx.x & 3;
+    const bool live = col < dv;
+    const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
+    const int slot = p.slots[seq];
+    if (slot < 0 || hi <= lo) return;                        // a padded row (uniform over the workgroup)
+    const bool fresh = p.context_lens[seq] == hi - lo;
+    float* sp = p.state + (((int64_t)slot * p.H + head) * dk) * dv;
+    float S[DKQ];
+#pragma unroll
+    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && ii < dkq) ? sp[(int64_t)(4 * ii + sub) * dv + col] : 0.f;
+    const int rowf = 5 * dk + dv, n = p.H * dk;
+    for (int t0 = lo; t0 < hi; t0 += DTOK) {
+        const int nt = min(DTOK, hi - t0);
+        __syncthreads();
+        for (int i = threadIdx.x; i < nt * rowf; i += 256) {
+            const int tt = i / rowf, e = i - tt * rowf;
+            const int64_t tok = t0 + tt;
+            float v;
+            if (e < dk) v = ldf((const A*)p.r, tok * p.r_stride + head * dk + e);
+            else if (e < 2 * dk) v = ldf((const A*)p.k, tok * p.k_stride + head * dk + e - dk);
+            else if (e < 5 * dk) v = p.wua[tok * 3 * n + (int64_t)((e - 2 * dk) / dk) * n + head * dk + (e - 2 * dk) % dk];
+            else v = ldf((const A*)p.v, tok * p.v_stride + head * dv + e - 5 * dk);
+            sm[i] = v;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float* row = sm + tt * rowf;
+            const float *rr = row, *kk = row + dk, *ww = row + 2 * dk, *uu = row + 3 * dk, *au = row + 4 * dk;
+            const float vj = live ? row[5 * dk + col] : 0.f;
+            float dot = 0.f;
+#pragma unroll
+            for (int ii = 0; ii < DKQ; ++ii)
+                if (ii < dkq) dot = __builtin_fmaf(uu[4 * ii + sub], S[ii], dot);
+            dot += NVH_DPP(dot, 0xB1);
+            dot += NVH_DPP(dot, 0x4E);
+            float o = 0.f;
+#pragma unroll
+            for (int ii = 0; ii < DKQ; ++ii)
+                if (ii < dkq) {
+                    const int i = 4 * ii + sub;
+                    const float s = __builtin_fmaf(ww[i], S[ii], __builtin_fmaf(kk[i], vj, -(au[i] * dot)));
+                    S[ii] = s;
+                    o = __builtin_fmaf(s, rr[i], o);
+                }
+            o += NVH_DPP(o, 0xB1);
+            o += NVH_DPP(o, 0x4E);
+            if (live && sub == 0) p.out[(int64_t)(t0 + tt) * p.H * dv + head * dv + col] = o;
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int ii = 0; ii < DKQ; ++ii)
+            if (ii < dkq) sp[(int64_t)(4 * ii + sub) * dv + col] = S[ii];
+    }
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void delta_post_kernel(const float* __restrict__ o, const A* __restrict__ norm_w, const A* __restrict__ gate,
+                                                         int64_t gate_stride, A* __restrict__ y, int64_t y_stride, int64_t rows, int H, int dv, float eps) {
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);     // (token, head) per wave
+    if (item >= rows * H) return;
+    const int64_t t = item / H;
+    const int h = (int)(item - t * H), lane = threadIdx.x & 63;
+    const float* orow = o + (t * H + h) * dv;
+    float ss = 0.f;
+    for (int i = lane; i < dv; i += 64) ss += orow[i] * orow[i];
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)dv + eps);
+    for (int i = lane; i < dv; i += 64) {
+        const int c = h * dv + i;
+        const float g = gate ? sigmoidf_(ldf(gate, t * gate_stride + c)) : 1.0f;
+        y[t * y_stride + c] = (A)(orow[i] * inv * ldf(norm_w, c) * g);
+    }
+}
+
+}  // namespace
+
+extern "C" int32_t nvh_delta_prep(const void* k, int64_t k_stride, const void* a_raw, int64_t a_stride, const void* lowrank, int64_t lowrank_stride,
+                                  const void* w2, const void* w0, const void* a_bias, float* out, int64_t num_tokens, int64_t heads, int64_t dk,
+                                  int64_t rank, float decay_scale, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(k && a_raw && lowrank && w2 && w0 && a_bias && out, NVH_EINVAL, "nvh_delta_prep: null pointer");
+    NVH_REQUIRE(num_tokens >= 0 && heads > 0 && dk > 0 && rank > 0 && rank <= 8192, NVH_EINVAL, "nvh_delta_prep: bad sizes");
+    if (num_tokens == 0) return NVH_OK;
+    DeltaPrepArgs p{k, k_stride, a_raw, a_stride, lowrank, lowrank_stride, w2, w0, a_bias, out, (int)heads, (int)dk, (int)rank, decay_scale};
+    hipStream_t st = (hipStream_t)stream;
+    const size_t lds = sizeof(float) * (size_t)rank;
+    if (act_f32) delta_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
+    else delta_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_delta_prep");
+    return NVH_OK;
+}
+
+template <typename A>
+static int32_t launch_delta_scan(const DeltaScanArgs& p, int64_t batch, hipStream_t st) {
+    const dim3 grid((unsigned)batch, (unsigned)p.H, (unsigned)nvh_cdiv(p.dv, 64));
+    const size_t lds = sizeof(float) * (size_t)DTOK * (5 * p.dk + p.dv);
+    const int dkq = p.dk / 4;
+    if (dkq <= 8) delta_scan_kernel<A, 8><<<grid, 256, lds, st>>>(p);
+    else if (dkq <= 16) delta_scan_kernel<A, 16><<<grid, 256, lds, st>>>(p);
+    else if (dkq <= 32) delta_scan_kernel<A, 32><<<grid, 256, lds, st>>>(p);
+    else delta_scan_kernel<A, 64><<<grid, 256, lds, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_delta_scan");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_delta_scan(const void* r, int64_t r_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                                  const float* wua, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                                  const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
+                                  int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(r && k && v && wua && state && slots && context_lens && out, NVH_EINVAL, "nvh_delta_scan: null pointer");
+    NVH_REQUIRE(batch >= 0 && heads > 0 && dk > 0 && dv > 0, NVH_EINVAL, "nvh_delta_scan: bad sizes");
+    NVH_REQUIRE(dk % 4 == 0 && dk <= 256, NVH_ENOSYS, "nvh_delta_scan: key size %ld must be a multiple of 4, at most 256", (long)dk);
+    if (batch == 0) return NVH_OK;
+    DeltaScanArgs p{r, k, v, r_stride, k_stride, v_stride, wua, state, slots, cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dv};
+    return act_f32 ? launch_delta_scan<float>(p, batch, (hipStream_t)stream) : launch_delta_scan<bf16>(p, batch, (hipStream_t)stream);
+}
+
+extern "C" int32_t nvh_delta_post(const float* o, const void* norm_weight, const void* gate, int64_t gate_stride, void* y, int64_t y_stride,
+                                  int64_t rows, int64_t heads, int64_t dv, float eps, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(o && norm_weight && y && rows >= 0 && heads > 0 && dv > 0, NVH_EINVAL, "nvh_delta_post: bad argument");
+    if (rows == 0) return NVH_OK;
+    const unsigned blocks = (unsigned)nvh_cdiv(rows * heads, 4);
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) delta_post_kernel<float><<<dim3(blocks), 256, 0, st>>>(o, (const float*)norm_weight, (const float*)gate, gate_stride, (float*)y, y_stride, rows, (int)heads, (int)dv, eps);
+    else delta_post_kernel<bf16><<<dim3(blocks), 256, 0, st>>>(o, (const bf16*)norm_weight, (const bf16*)gate, gate_stride, (bf16*)y, y_stride, rows, (int)heads, (int)dv, eps);
+    NVH_CHECK_LAUNCH("nvh_delta_post");
+    return NVH_OK;
+}

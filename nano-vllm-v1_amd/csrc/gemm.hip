@@ -363,7 +363,8 @@ __global__ __launch_bounds__(64 * WAVES_N * WAVES_M) void gemm_bf16_nt_kernel(
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
             const int m = m0 + wm * WM + j * 16 + fr;
-            const float inv_t = 1.0f / se.temps[min(m, M - 1)];
+            const float t_row = se.temps[min(m, M - 1)];
+            const float inv_t = t_row > 0.f ? 1.0f / t_row : 0.f;
             best[j] = ValIdx{-INFINITY, (int64_t)0x7fffffffffffffffLL};
 #pragma unroll
             for (int i = 0; i < TN; ++i) {                       // increasing columns: "strictly greater" keeps the lowest index

@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void sample_slice_kernel(const void* __restric
     float t = 1.f, inv_t = 1.f;
     if constexpr (MODE != 0) {
         t = temps[row];
-        inv_t = 1.0f / t;
+        inv_t = t > 0.f ? 1.0f / t : 0.f;                    // 0: greedy (nvh_race_scores)
     }
     // The lane scans increasing indices, so "strictly greater" keeps the lowest index among equals; the index stays
     // 32-bit (relative to the slice start) until the cross-lane reduction.

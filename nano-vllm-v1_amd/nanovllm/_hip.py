@@ -88,6 +88,20 @@ SIGNATURES = {
     "nvh_qwen3_forward_parts": (i32, [vp, vp, vp, vp, i64, i32, i32, vp]),
     "nvh_qwen3_exchange_buffers": (i32, [vp, i64, i64, i32, vp, vp, vp]),
     "nvh_qwen3_logits": (i32, [vp, vp, vp, vp, i64, vp, vp, vp]),
+    # operators with an fp32 residual stream, free head sizes and a choice of activation type (csrc/stream_f32.hip,
+    # attention_any.hip, delta_rule.hip)
+    "nvh_embedding_stream": (i32, [vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]),
+    "nvh_residual_dyt": (i32, [vp, i64, vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, i64, i64, i64, i32, vp]),
+    "nvh_stream_cast": (i32, [vp, vp, i64, i64, i64, i32, vp]),
+    "nvh_gelu_tanh_mul": (i32, [vp, i64, vp, i64, i64, i32, vp]),
+    "nvh_gather_rows_f32": (i32, [vp, vp, vp, i64, i64, vp]),
+    "nvh_logit_softcap": (i32, [vp, i64, vp, i64, i64, f32, i32, vp]),
+    "nvh_gemm_any_nt": (i32, [vp, i64, vp, vp, vp, i64, i64, i64, i64, i32, i32, vp]),
+    "nvh_attn_rotary_prep": (i32, [vp, i64, vp, vp, f32, vp, vp, f32, i64, i32, vp, i32, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i32, vp]),
+    "nvh_attn_paged_any": (i32, [vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, i64, f32, vp, vp, i32, vp, i32, vp]),
+    "nvh_delta_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, i64, i64, i64, i64, f32, i32, vp]),
+    "nvh_delta_scan": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]),
+    "nvh_delta_post": (i32, [vp, vp, vp, i64, vp, i64, i64, i64, i64, f32, i32, vp]),
 }
 
 _lib = None

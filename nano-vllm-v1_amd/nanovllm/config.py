@@ -4,6 +4,9 @@ read step n's sampled ids, so the GPU never waits for the host between steps.  S
 to what depends on WHEN a value is seen (eos ends a sequence one step later: the token computed past it is dropped);
 ``async_scheduling=False`` runs the reference's loop (engine/llm_engine.py:117-126): schedule, run, read ids, postprocess.
 
+``dtype`` and ``num_state_slots`` are not in the reference either: the activation type a model is served in (models
+that support fp32 run every product in true 32-bit then) and the number of recurrent-state slots.
+
 ``model`` is a local directory holding a Hugging Face ``config.json`` (and optionally
 ``*.safetensors`` weights; without them the runner initialises synthetic weights).
 """
@@ -18,15 +21,20 @@ import torch
 
 
 def load_hf_config(path: str):
-    """AutoConfig when transformers is importable, else the raw config.json as a namespace."""
-    try:
-        from transformers import AutoConfig
-        return AutoConfig.from_pretrained(path)
-    except ImportError:
-        with open(os.path.join(path, "config.json")) as f:
-            raw = json.load(f)
-        raw["torch_dtype"] = getattr(torch, raw.get("torch_dtype", "bfloat16"))
-        return SimpleNamespace(**raw)
+    """config.json of a model directory.  A config that names a `model_type` goes through transformers' AutoConfig when it
+    is importable; any other (a design that no library knows: it names its `architecture` itself) is the raw JSON as a
+    namespace, nested objects left as dicts."""
+    with open(os.path.join(path, "config.json")) as f:
+        raw = json.load(f)
+    if "model_type" in raw:
+        try:
+            from transformers import AutoConfig
+            return AutoConfig.from_pretrained(path)
+        except ImportError:
+            pass
+    if isinstance(raw.get("torch_dtype"), str):
+        raw["torch_dtype"] = getattr(torch, raw["torch_dtype"])
+    return SimpleNamespace(**raw)
 
 
 def model_dtype(hf_config) -> torch.dtype:
@@ -49,6 +57,10 @@ class Config:
     num_kvcache_blocks: int = -1
     chunked_prefill: bool = False
     async_scheduling: bool = True
+    dtype: str | None = None            # "bfloat16" / "float32": serve the model in this type instead of its checkpoint's (None)
+    num_state_slots: int = -1           # recurrent-state slots (models with a per-sequence state); -1: one per max_num_seqs
+    prefix_caching: bool = True         # share resident pages between prompts with a common prefix (off for recurrent models)
+    recurrent_state: bool = False       # set by the runner: the loaded model keeps a state per sequence
 
     def __post_init__(self):
         # the reference asserts a multiple of 256 (config.py:82) but its Sequence.block_size is the constant 256
@@ -57,4 +69,7 @@ class Config:
         assert 1 <= self.tensor_parallel_size <= 8
         if self.hf_config is None:
             self.hf_config = load_hf_config(self.model)
-        self.max_model_len = min(self.max_model_len, self.hf_config.max_position_embeddings)
+        # (a design whose positions no table bounds has no max_position_embeddings: max_model_len stands as given)
+        self.max_model_len = min(self.max_model_len, getattr(self.hf_config, "max_position_embeddings", None) or self.max_model_len)
+        if self.num_state_slots <= 0:
+            self.num_state_slots = self.max_num_seqs

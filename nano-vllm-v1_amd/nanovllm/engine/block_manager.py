@@ -63,8 +63,17 @@ class _FreeList:
 
 
 class BlockManager:
-    def __init__(self, num_blocks: int, block_size: int):
+    """Pages and, for models whose layers carry a recurrent state, state slots: a sequence takes one slot when it is
+    admitted and gives it back with its pages (`num_state_slots` 0: the model has no such state).  A slot's content is
+    never cleared here: a sequence whose first tokens are scheduled starts from a zero state on the device.  With a
+    recurrent state a resident page cannot stand in for a prefix (the state after it is gone), so such models run with
+    `prefix_caching` off: no page is hashed or shared."""
+
+    def __init__(self, num_blocks: int, block_size: int, num_state_slots: int = 0, prefix_caching: bool = True):
         self.block_size = block_size
+        self.prefix_caching = prefix_caching
+        self.num_state_slots = num_state_slots
+        self.free_state_slots = list(range(num_state_slots - 1, -1, -1))     # a stack: the slot released last is handed out first
         self.blocks = [Block(i) for i in range(num_blocks)]
         self.hash_to_block_id: dict[int, int] = {}
         self.free_block_ids = _FreeList(range(num_blocks))
@@ -88,6 +97,9 @@ class BlockManager:
         h = NO_HASH
         for i in range(seq.num_blocks):
             tokens = seq.block(i)
+            if not self.prefix_caching:
+                yield i, tokens, NO_HASH, -1
+                continue
             h = self.compute_hash(tokens, h) if len(tokens) == self.block_size else NO_HASH
             page = self.hash_to_block_id.get(h, -1)
             if page != -1 and self.blocks[page].token_ids != tokens:
@@ -121,6 +133,8 @@ class BlockManager:
 
     # ------------------------------------------------------------------ admission of a waiting sequence
     def can_allocate(self, num_tokens: int) -> bool:
+        if self.num_state_slots and not self.free_state_slots:
+            return False
         return len(self.free_block_ids) >= self._pages_for(num_tokens)
 
     def get_token_layout(self, seq: Sequence) -> tuple[int, int, int]:
@@ -141,6 +155,8 @@ class BlockManager:
     def allocate(self, seq: Sequence):
         """Give `seq` its shared prefix pages, then fresh pages for the seq.num_new_tokens scheduled tokens."""
         assert not seq.block_table
+        if self.num_state_slots:
+            seq.state_slot = self.free_state_slots.pop()
         bs = self.block_size
         h = NO_HASH
         for _, tokens, h, page in self._chain(seq):
@@ -159,7 +175,7 @@ class BlockManager:
         for lo in range(first, end, bs):
             tokens = seq[lo:min(lo + bs, end)]
             if lo != first:
-                h = self.compute_hash(tokens, h) if len(tokens) == bs else NO_HASH
+                h = self.compute_hash(tokens, h) if len(tokens) == bs and self.prefix_caching else NO_HASH
             block = self._take(self.free_block_ids[0])
             if h != NO_HASH and len(tokens) == bs:
                 self._label(block, h, tokens)
@@ -167,6 +183,9 @@ class BlockManager:
 
     def deallocate(self, seq: Sequence):
         self.deferred.pop(seq.seq_id, None)
+        if seq.state_slot >= 0:
+            self.free_state_slots.append(seq.state_slot)
+            seq.state_slot = -1
         for page in reversed(seq.block_table):
             block = self.blocks[page]
             block.ref_count -= 1
@@ -197,7 +216,7 @@ class BlockManager:
             if block is None:
                 block = self._take(self.free_block_ids[0])
                 seq.block_table.append(block.block_id)
-            if len(tokens) == bs:
+            if len(tokens) == bs and self.prefix_caching:
                 if tokens[-1] == PLACEHOLDER:
                     self.deferred[seq.seq_id] = (seq, index)     # hashed when the id arrives
                     continue

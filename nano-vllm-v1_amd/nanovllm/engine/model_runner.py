@@ -32,11 +32,12 @@ import torch.distributed as dist
 from .. import _hip, comm
 from ..config import Config, model_dtype
 from ..layers.sampler import Sampler
+from ..models import get_model_class
 from ..models.qwen3 import Qwen3ForCausalLM
 from ..native import MODE_DECODE, MODE_PACKED, MODE_PAGED, NativeQwen3
 from .. import ops
 from ..utils.context import get_context, reset_context, set_context
-from ..utils.loader import has_checkpoint, load_model, load_tensors, synthetic_tensors
+from ..utils.loader import checkpoint_shapes, has_checkpoint, load_model, load_tensors, synthetic_tensors
 from .sequence import Sequence
 
 try:
@@ -195,6 +196,7 @@ class ModelRunner:
         self._lane_done = {}                    # side lane -> completion event of the last step launched on it
         self._recent_steps = collections.deque()   # completion events of the steps launched last (bounds the run-ahead)
         self._step_depth, self._step_fb = 0, None
+        self._want_rows = None                  # forward_logits(rows=...): flat token rows of the step whose logits are asked for
         self.comm = None
         if self.world_size > 1:
             # staging: the widest all-reduce (a full token budget of hidden rows) or logits gather (every sequence)
@@ -210,16 +212,32 @@ class ModelRunner:
                 if dist.get_backend() != "nccl":
                     self.enforce_eager = True
 
-        dtype = model_dtype(hf)
-        if dtype != torch.bfloat16:
-            raise _hip.HipError(f"model dtype {dtype} unsupported: the kernel path is bf16 only")
+        # The model class comes from the registry (config.json names the architecture).  The Qwen3 family runs the bf16 kernel
+        # path with its native executor; any other class runs as operator modules over the kernels it names itself, in
+        # the activation types it lists (`generic`: everything below that is not Qwen3-specific).
+        cls = get_model_class(hf)
+        dtype = getattr(torch, config.dtype) if config.dtype else model_dtype(hf)
+        if dtype not in getattr(cls, "supported_dtypes", (torch.bfloat16,)):
+            raise _hip.HipError(f"model dtype {dtype} unsupported by {cls.__name__}: its kernel path runs "
+                                f"{', '.join(str(d) for d in getattr(cls, 'supported_dtypes', (torch.bfloat16,)))}")
+        self.dtype = dtype
+        self.generic = cls is not Qwen3ForCausalLM
+        self.always_paged = bool(getattr(cls, "requires_cache", False))
+        config.recurrent_state = bool(getattr(cls, "has_recurrent_state", False))
+        if self.generic:
+            assert self.world_size == 1, f"{cls.__name__} is served on one GPU (its layers are not tensor-parallel)"
+            self.enforce_eager = True            # its steps are launched one by one (no captured decode graph yet)
         prev_dtype = torch.get_default_dtype()
         torch.set_default_dtype(dtype)
         torch.set_default_device(self.device)
         try:
-            self.model = Qwen3ForCausalLM(hf)
+            if hasattr(cls, "adapt_config"):
+                cls.adapt_config(hf, checkpoint_shapes(config.model) if has_checkpoint(config.model) else {})
+            self.model = cls(hf)
             if has_checkpoint(config.model):
                 load_model(self.model, config.model)
+            elif hasattr(cls, "synthetic_tensors"):
+                load_tensors(self.model, cls.synthetic_tensors(hf, seed=0, device=self.device, dtype=dtype))
             else:
                 load_tensors(self.model, synthetic_tensors(hf, seed=0, device=self.device, dtype=dtype))
             self.sampler = Sampler()
@@ -228,7 +246,7 @@ class ModelRunner:
             # one native call per step (per rank; ranks meet through the xGMI exchange); the operator modules,
             # with torch.distributed collectives between them when the exchange is unavailable, otherwise.
             # NANOVLLM_NATIVE=0 forces the module path (parity tests use it).
-            use_native = os.environ.get("NANOVLLM_NATIVE", "1") != "0" and not getattr(hf, "attention_bias", True)
+            use_native = not self.generic and os.environ.get("NANOVLLM_NATIVE", "1") != "0" and not getattr(hf, "attention_bias", True)
             external_sum = comm.all_reduce if (self.world_size > 1 and self.comm is None) else None
             self.native = NativeQwen3(self.model, comm=self.comm, reduce_fn=external_sum) if use_native else None
             # tensor-parallel ranks sample over their vocabulary shards instead of gathering the logits on rank 0
@@ -344,7 +362,8 @@ class ModelRunner:
 
     # -------------------------------------------------------------- init-time passes
     def warmup_model(self):
-        """One maximum-shape forward without a cache, to measure peak activation memory."""
+        """One maximum-shape forward without a cache, to measure peak activation memory (a model that always reads paged
+        caches gets a pool of just the pages this forward needs, released afterwards)."""
         torch.cuda.empty_cache()
         torch.cuda.reset_peak_memory_stats()
         cfg = self.config
@@ -353,9 +372,49 @@ class ModelRunner:
         seqs = [Sequence([0] * length) for _ in range(num_seqs)]
         for seq in seqs:
             seq.num_new_tokens = length
+        if self.always_paged:
+            per_seq = -(-length // self.block_size)
+            self._bind_generic_caches(num_seqs * per_seq, num_seqs)
+            for i, seq in enumerate(seqs):
+                seq.block_table = list(range(i * per_seq, (i + 1) * per_seq))
+                seq.state_slot = i
         self.run(seqs)
         torch.cuda.synchronize()
+        if self.always_paged:
+            self._bind_generic_caches(0, 0)
         torch.cuda.empty_cache()
+
+    # -------------------------------------------------------------- caches of models that describe their own
+    def _cache_modules(self):
+        """(attention modules with page caches, recurrent modules with state pools) of a generic model."""
+        paged = [m for m in self.model.modules() if hasattr(m, "k_caches") and hasattr(m, "cache_row_elems")]
+        recurrent = [m for m in self.model.modules() if hasattr(m, "states") and hasattr(m, "state_shape")]
+        return paged, recurrent
+
+    def generic_block_bytes(self) -> int:
+        itemsize = torch.empty(0, dtype=self.dtype).element_size()
+        paged, _ = self._cache_modules()
+        return sum(m.cache_runs * self.block_size * sum(m.cache_row_elems()) * itemsize for m in paged)
+
+    def generic_state_bytes(self, slots: int) -> int:
+        _, recurrent = self._cache_modules()
+        return sum(m.state_runs * slots * int(np.prod(m.state_shape())) * 4 for m in recurrent)
+
+    def _bind_generic_caches(self, num_blocks: int, slots: int):
+        """Page caches [blocks, page, G, dim | vdim] per attention module and pass, fp32 state pools [slots, ...] per recurrent
+        module and pass (num_blocks 0: release them).  Nothing is cleared beyond allocation: keys are written before they are
+        read, and a sequence's state is taken as zero in the step that brings its first tokens."""
+        paged, recurrent = self._cache_modules()
+        for m in paged:
+            for run in range(m.cache_runs):
+                if num_blocks:
+                    m.k_caches[run] = torch.zeros(num_blocks, self.block_size, m.num_kv_heads, m.head_dim, dtype=self.dtype, device=self.device)
+                    m.v_caches[run] = torch.zeros(num_blocks, self.block_size, m.num_kv_heads, m.value_dim, dtype=self.dtype, device=self.device)
+                else:
+                    m.k_caches[run] = m.v_caches[run] = None
+        for m in recurrent:
+            for run in range(m.state_runs):
+                m.states[run] = torch.zeros(slots, *m.state_shape(), dtype=torch.float32, device=self.device) if slots else None
 
     def kv_block_bytes(self) -> int:
         hf = self.config.hf_config
@@ -368,6 +427,17 @@ class ModelRunner:
         A positive ``config.num_kvcache_blocks`` is honoured (tests, benchmarks); otherwise the pool
         takes what ``gpu_memory_utilization`` leaves after weights and peak activations."""
         cfg, hf = self.config, self.config.hf_config
+        if self.generic:
+            slots = cfg.num_state_slots if cfg.recurrent_state else 0
+            if cfg.num_kvcache_blocks <= 0:
+                free, total = torch.cuda.mem_get_info()
+                stats = torch.cuda.memory_stats()
+                peak, current = stats["allocated_bytes.all.peak"], stats["allocated_bytes.all.current"]
+                room = int(total * cfg.gpu_memory_utilization - (total - free) - peak + current) - self.generic_state_bytes(slots)
+                cfg.num_kvcache_blocks = room // max(self.generic_block_bytes(), 1)
+            assert cfg.num_kvcache_blocks > 0
+            self._bind_generic_caches(cfg.num_kvcache_blocks, slots)
+            return
         if cfg.num_kvcache_blocks <= 0:
             free, total = torch.cuda.mem_get_info()
             used = total - free
@@ -394,6 +464,10 @@ class ModelRunner:
                                      "context_lens", "need")}
         if fb["block_tables"] is not None:
             arrays["block_tables"] = fb["block_tables"]
+        if self.config.recurrent_state:
+            arrays["state_slots"] = np.fromiter((s.state_slot for s in seqs), dtype=np.int32, count=len(seqs))
+        if fb.get("logit_rows") is not None:
+            arrays["logit_rows"] = fb["logit_rows"]
         if self.rank == 0 or self.shard_sampling:
             temps = np.fromiter((s.temperature for s in seqs), dtype=np.float32, count=len(seqs))
             arrays["temperatures"] = temps[fb["need"]] if fb["need"].size else temps
@@ -430,7 +504,8 @@ class ModelRunner:
         fb["items"] = None if plan is None else {k: d[k] for k in ("item_seq", "item_range", "seq_active", "seq_chunk")}
         fb["tails"] = (d.get("cu_seqlens_q_tail"), d.get("cu_seqlens_k_tail"))
         set_context(d["cu_seqlens_q"], d["cu_seqlens_k"], fb["max_seqlen_q"], fb["max_seqlen_k"], d["slot_mapping"],
-                    d["context_lens"], d.get("block_tables"), d["need"])
+                    d["context_lens"], d.get("block_tables"), d["need"], d.get("state_slots"))
+        fb["logit_rows_dev"] = d.get("logit_rows")
         return d["input_ids"], d["positions"], d.get("temperatures"), fb
 
     # -------------------------------------------------------------- forward
@@ -508,7 +583,7 @@ class ModelRunner:
     def _graph_for(self, fb):
         """The captured graph that fits this step, or None (eager)."""
         bs = len(fb["context_lens"])
-        if (self.enforce_eager or not self.graphs or fb["block_tables"] is None or fb["max_seqlen_q"] != 1
+        if (self.enforce_eager or not self.graphs or fb["block_tables"] is None or fb["max_seqlen_q"] != 1 or fb.get("logit_rows") is not None
                 or fb["input_ids"].size != bs or fb["need"].size != bs or bs > self.graph_bs[-1]
                 or fb["block_tables"].shape[1] > self.graph_width):
             return None
@@ -554,6 +629,14 @@ class ModelRunner:
         while len(self._recent_steps) >= max(self.LANES, 2):   # (two: what the loop that runs one step ahead needs)
             self._recent_steps.popleft().synchronize()
         fb = flatten_batch(seqs, self.block_size)
+        if self.always_paged and fb["block_tables"] is None and len(seqs):
+            # a step without cached keys still goes through the pages: this model has no packed mode
+            width = max(len(s.block_table) for s in seqs)
+            tables = np.full((len(seqs), max(width, 1)), -1, dtype=np.int32)
+            for i, sq in enumerate(seqs):
+                tables[i, :len(sq.block_table)] = sq.block_table
+            fb["block_tables"] = tables
+        fb["logit_rows"] = self._want_rows
         fb["fed"] = self._fed_indices(seqs, fb)
         fb["graph"] = self._graph_for(fb)
         last = self._last_step
@@ -607,8 +690,20 @@ class ModelRunner:
             input_ids, positions, temps, _ = self.prepare_model_input(seqs, fb)
             hidden = self.forward_hidden(input_ids, positions, fb)
             ctx = get_context()
-            if fb["need"].size == 0 and any(len(s.block_table) for s in seqs):
+            if fb.get("logit_rows") is not None:
+                # explicit rows (any positions of the step, not only the last of a sequence): selected here, projected as they are
+                idx = fb["logit_rows_dev"]
+                picked = self.model.gather_rows(hidden, idx) if hasattr(self.model, "gather_rows") else hidden.index_select(0, idx.long())
+                out = (picked, None, None, picked.shape[0], temps, need_host)
+            elif fb["need"].size == 0 and any(len(s.block_table) for s in seqs):
                 out = (hidden, None, None, 0, temps, need_host)
+            elif hasattr(self.model, "gather_rows"):
+                # the last row of every sequence that ends its scheduled tokens here (all sequences when none owns pages)
+                cu = fb["cu_seqlens_q"]
+                last = (cu[1:][fb["need"]] if fb["need"].size else cu[1:]) - 1
+                idx = torch.from_numpy(np.ascontiguousarray(last, dtype=np.int32)).to(self.device, non_blocking=True)
+                rows = self.model.gather_rows(hidden, idx)
+                out = (rows, None, None, rows.shape[0], temps, need_host)
             elif self.native is not None:
                 out = (hidden, ctx.cu_seqlens_q, ctx.seq_need_compute_logits if fb["need"].size else None,
                        fb["need"].size or len(seqs), temps, need_host)
@@ -620,19 +715,30 @@ class ModelRunner:
         return out
 
     @torch.inference_mode()
-    def forward_logits(self, seqs, gather=True):
+    def _logits_of_rows(self, rows):
+        if hasattr(self.model, "compute_logits_rows"):
+            return self.model.compute_logits_rows(rows)
+        return self.model.lm_head.forward_rows(rows)
+
+    def forward_logits(self, seqs, gather=True, rows=None):
         """Everything of a step up to the sampler: (logits [B', V] | None, temperatures | None, need)
         with ``need`` a HOST int32 tensor (indices into ``seqs`` of the rows of ``logits``).  logits is
         None on ranks > 0 and when no sequence finishes its scheduled prompt in this step.  ``gather=False`` (tensor
-        parallelism with the native executor): every rank keeps the logits of ITS vocabulary shard, [B', V / tp]."""
-        with self._step(seqs, join=True):
-            hidden, cu, keep, n, temps, need_host = self._forward_rows(seqs, self.rank == 0 or not gather)
-            if n == 0:
-                logits = None
-            elif self.native is not None:
-                logits = self.native.logits(hidden, cu, keep, n, gather=gather)
-            else:
-                logits = self.model.lm_head.forward_rows(hidden)
+        parallelism with the native executor): every rank keeps the logits of ITS vocabulary shard, [B', V / tp].
+        ``rows`` (int32 array; not in the reference): logits of these rows of the step's packed tokens instead - any
+        positions, e.g. every prompt token of a scoring run - in the given order; the step runs eagerly then."""
+        self._want_rows = None if rows is None else np.ascontiguousarray(rows, dtype=np.int32)
+        try:
+            with self._step(seqs, join=True):
+                hidden, cu, keep, n, temps, need_host = self._forward_rows(seqs, self.rank == 0 or not gather)
+                if n == 0:
+                    logits = None
+                elif self.native is not None:
+                    logits = self.native.logits(hidden, cu, keep, n, gather=gather)
+                else:
+                    logits = self._logits_of_rows(hidden)
+        finally:
+            self._want_rows = None
         return logits, temps, need_host
 
     @torch.inference_mode()

@@ -30,7 +30,11 @@ class Scheduler:
         self.max_num_seqs = config.max_num_seqs
         self.max_num_batched_tokens = config.max_num_batched_tokens
         self.eos = config.eos
-        self.block_manager = BlockManager(config.num_kvcache_blocks, config.kvcache_block_size)
+        # (recurrent_state / prefix_caching: what the runner found out about the model it loaded)
+        recurrent = getattr(config, "recurrent_state", False)
+        self.block_manager = BlockManager(config.num_kvcache_blocks, config.kvcache_block_size,
+                                          num_state_slots=getattr(config, "num_state_slots", 0) if recurrent else 0,
+                                          prefix_caching=getattr(config, "prefix_caching", True) and not recurrent)
         self.waiting: deque[Sequence] = deque()
         self.running: deque[Sequence] = deque()
         self.num_preemptions = 0            # bookkeeping for the serving harness; scheduling never reads it
@@ -186,3 +190,42 @@ class Scheduler:
             elif seq.status == SequenceStatus.RUNNING:
                 self.block_manager.label_deferred(seq)
         return done
+
+    # ------------------------------------------------------------------ a schedule dictated from outside
+    def replay_step(self, live: dict, request_id, tokens: list[int]) -> Sequence:
+        """The next `tokens` of request `request_id` are to run in the coming step, whatever this scheduler would have
+        chosen (replay of a recorded schedule, scoring of given text): admits the request at its first tokens (pages for
+        them, a state slot), extends it otherwise, and returns its sequence with `num_new_tokens` set.  `live` maps the
+        caller's request ids to their sequences."""
+        bm = self.block_manager
+        seq = live.get(request_id)
+        if seq is None:
+            seq = Sequence(list(tokens))
+            seq.num_new_tokens = len(tokens)
+            if len(self.running) >= self.max_num_seqs or not bm.can_allocate(len(tokens)):
+                raise RuntimeError(f"request {request_id!r}: no room for {len(tokens)} tokens ({len(bm.free_block_ids)} pages free, "
+                                   f"{len(self.running)} of {self.max_num_seqs} requests live)")
+            bm.allocate(seq)
+            seq.status = SequenceStatus.RUNNING
+            self.running.append(seq)
+            live[request_id] = seq
+            return seq
+        for t in tokens:
+            seq.append_token(t)
+        if not bm.can_append(seq, len(tokens)):
+            raise RuntimeError(f"request {request_id!r}: no pages left for {len(tokens)} more tokens")
+        seq.num_new_tokens = len(tokens)
+        bm.may_append(seq)
+        return seq
+
+    def replay_done(self, seqs: list[Sequence]) -> None:
+        """The step has been launched: its tokens are now cached ones."""
+        for seq in seqs:
+            seq.num_cached_tokens += seq.num_new_tokens
+            seq.num_new_tokens = 0
+
+    def replay_end(self, live: dict, request_id) -> None:
+        seq = live.pop(request_id)
+        seq.status = SequenceStatus.FINISHED
+        self.block_manager.deallocate(seq)
+        self.running.remove(seq)

@@ -38,6 +38,7 @@ class Sequence:
         self.max_tokens = sp.max_tokens
         self.ignore_eos = sp.ignore_eos
         self.pending_slot = -1              # row of the newest placeholder's id in the sampler output it will come from
+        self.state_slot = -1                # recurrent-state slot while the sequence is running (models with such a state)
 
     def __len__(self):
         return self.num_tokens
@@ -87,11 +88,11 @@ class Sequence:
     def __getstate__(self):
         lo, hi = self.num_cached_tokens, self.num_cached_tokens + self.num_new_tokens
         return (self.num_tokens, self.num_prompt_tokens, self.num_cached_tokens, self.num_new_tokens,
-                self.block_table, self.temperature, lo, self.token_ids[lo:hi], self.pending_slot)
+                self.block_table, self.temperature, lo, self.token_ids[lo:hi], self.pending_slot, self.state_slot)
 
     def __setstate__(self, state):
         (self.num_tokens, self.num_prompt_tokens, self.num_cached_tokens, self.num_new_tokens,
-         self.block_table, self.temperature, lo, window, self.pending_slot) = state
+         self.block_table, self.temperature, lo, window, self.pending_slot, self.state_slot) = state
         self.token_ids = _Window(lo, window, self.num_tokens)
         self.last_token = window[-1] if window else -1
 

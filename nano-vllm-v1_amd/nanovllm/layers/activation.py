@@ -1,5 +1,6 @@
-"""SwiGLU gate: silu(x[..., :I]) * x[..., I:] (reference: nanovllm/layers/activation.py:36-58);
-kernel nvh_silu_mul in csrc/elementwise.hip."""
+"""Gated activations over a merged [gate | up] projection: SwiGLU, silu(x[..., :I]) * x[..., I:] (reference:
+nanovllm/layers/activation.py:36-58; kernel nvh_silu_mul in csrc/elementwise.hip), and its GELU counterpart with the
+tanh form of GELU (kernel nvh_gelu_tanh_mul in csrc/stream_f32.hip; bf16 or fp32 rows)."""
 import torch
 from torch import nn
 
@@ -9,3 +10,10 @@ from .. import ops
 class SiluAndMul(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         return ops.silu_mul(x)
+
+
+class GeluTanhAndMul(nn.Module):
+    """gelu_tanh(x[..., :I]) * x[..., I:], gelu_tanh(z) = z/2 (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))), evaluated in fp32."""
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return ops.gelu_tanh_mul(x)

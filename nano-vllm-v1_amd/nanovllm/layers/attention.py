@@ -62,3 +62,45 @@ class Attention(nn.Module):
         if self.k_cache.numel() and self.v_cache.numel() and ctx.slot_mapping is not None and ctx.slot_mapping.numel():
             store_kvcache(k, v, self.k_cache, self.v_cache, ctx.slot_mapping)
         return self.attend(q, k, v)
+
+
+class GatedValueRotaryAttention(nn.Module):
+    """Paged causal attention with free head sizes (query/key `head_dim`, value `value_dim`), a partial rotary on q/k
+    whose frequencies the caller supplies, optionally values that are rotated by their own position before they are
+    cached (each head's output is turned back by the query's position), and optionally a per-head sigmoid output gate.
+
+    Input is the fused projection output [T, H*dim + G*dim + G*vdim (+ H)] = q | k | v | gate; RMS norms over the WHOLE
+    q and k projections run with the rotary in one launch (nvh_attn_rotary_prep), attention in a second
+    (nvh_attn_paged_any).  A module that serves several passes of a looped stack owns one cache per pass:
+    `k_caches[run]`, `v_caches[run]`, views [pages, page, G, dim|vdim] bound by the runner (`cache_runs` of them)."""
+
+    def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float, eps: float,
+                 rot_dims: int, qk_freq: torch.Tensor, qk_mag: float, value_freq: torch.Tensor | None, gated: bool,
+                 cache_runs: int = 1, interleaved: bool = False):
+        super().__init__()
+        assert num_heads % num_kv_heads == 0
+        self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim = num_heads, num_kv_heads, head_dim, value_dim
+        self.scale, self.eps, self.rot_dims, self.qk_mag, self.gated, self.interleaved = scale, eps, rot_dims, qk_mag, gated, interleaved
+        self.q_norm = nn.Parameter(torch.ones(num_heads * head_dim), requires_grad=False)
+        self.k_norm = nn.Parameter(torch.ones(num_kv_heads * head_dim), requires_grad=False)
+        self.register_buffer("qk_freq", qk_freq.to(dtype=torch.float32, device=self.q_norm.device), persistent=False)
+        self.register_buffer("value_freq", None if value_freq is None else value_freq.to(dtype=torch.float32, device=self.q_norm.device),
+                             persistent=False)
+        self.cache_runs = cache_runs
+        self.k_caches: list = [None] * cache_runs
+        self.v_caches: list = [None] * cache_runs
+
+    def cache_row_elems(self) -> tuple[int, int]:
+        """Elements of one token's key row and value row (what the runner sizes the page pool with)."""
+        return self.num_kv_heads * self.head_dim, self.num_kv_heads * self.value_dim
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, run: int = 0) -> torch.Tensor:
+        ctx = get_context()
+        kc, vc = self.k_caches[run], self.v_caches[run]
+        if kc is None or ctx.block_tables is None:
+            raise RuntimeError("this attention reads its keys from the paged cache: bind caches and give every sequence a block table")
+        q, gate = ops.attn_rotary_prep(proj, self.q_norm.data, self.k_norm.data, self.eps, positions, self.qk_freq, self.qk_mag,
+                                       self.rot_dims, self.value_freq, kc, vc, ctx.slot_mapping, self.num_heads, self.num_kv_heads,
+                                       self.head_dim, self.value_dim, self.gated, self.interleaved, self.interleaved)
+        return ops.attn_paged_any(q, kc, vc, ctx.cu_seqlens_q, ctx.context_lens, ctx.block_tables, self.scale, self.num_heads,
+                                  self.num_kv_heads, self.head_dim, self.value_dim, gate, self.value_freq, self.interleaved)

@@ -1,4 +1,6 @@
-"""RMSNorm operator module; arithmetic in csrc/elementwise.hip (nvh_rmsnorm / nvh_add_rmsnorm).
+"""Norm operator modules.  RMSNorm: arithmetic in csrc/elementwise.hip (nvh_rmsnorm / nvh_add_rmsnorm).
+DynamicTanh: a norm without statistics, tanh(alpha x) * weight + bias, applied together with the residual add around
+it by nvh_residual_dyt (csrc/stream_f32.hip) over an fp32 residual stream.
 
 Interface of the reference's nanovllm/layers/layernorm.py:48-165: ``RMSNorm(hidden_size,
 eps)``, ``.weight``, ``forward(x)`` -> y, ``forward(x, residual)`` -> (y, new_residual).
@@ -26,3 +28,24 @@ class RMSNorm(nn.Module):
         if slabs is not None:
             return ops.add_rmsnorm(None, residual, self.weight.data, self.eps, partials=slabs)
         return ops.add_rmsnorm(x, residual, self.weight.data, self.eps)
+
+
+class DynamicTanh(nn.Module):
+    """tanh(alpha * x) * weight + bias with a learned scalar alpha; no mean, no variance, no epsilon.
+
+    The module holds the parameters; the arithmetic runs fused with a residual add (ops.residual_dyt), which takes the
+    `triple()` of the norm after the sublayer and of the norm that opens the next one."""
+
+    def __init__(self, hidden_size: int, alpha: float = 0.5) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.ones(hidden_size), requires_grad=False)
+        self.bias = nn.Parameter(torch.zeros(hidden_size), requires_grad=False)
+        self.alpha = nn.Parameter(torch.full((1,), alpha), requires_grad=False)
+        self.alpha.weight_loader = lambda param, t: param.data.copy_(t.reshape(1))
+
+    def triple(self):
+        return self.alpha.data, self.weight.data, self.bias.data
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x fp32 [rows, dim] -> normalised rows in the parameters' type (x is left as it is)."""
+        return ops.residual_dyt(x, nxt=self.triple())

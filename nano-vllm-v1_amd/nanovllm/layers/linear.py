@@ -145,3 +145,33 @@ class RowParallelLinear(LinearBase):
         if self.tp_size > 1:
             y = comm.all_reduce(y)
         return y
+
+
+class MergedLinear(nn.Module):
+    """Several matrices that read the same input, stored as one weight [sum(out), in] and applied in one product of any
+    shape and either activation type (ops.linear_any: the tuned bf16 GEMM where its alignment rules hold, the any-shape
+    kernel otherwise).  Shards are named (`names[i]`); `split(y)` hands back the column views in order.  One rank only."""
+
+    def __init__(self, input_size: int, output_sizes: list[int], names: list | None = None):
+        super().__init__()
+        assert tp_world() == 1, "MergedLinear is not tensor-parallel"
+        self.output_sizes = list(output_sizes)
+        self.shard_ids = list(names) if names is not None else list(range(len(output_sizes)))
+        self.weight = nn.Parameter(torch.empty(sum(output_sizes), input_size), requires_grad=False)
+        self.weight.weight_loader = self.weight_loader
+        self.weight.shard_ids = self.shard_ids
+
+    def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor, loaded_shard_id=None):
+        if loaded_shard_id is None:
+            assert len(self.output_sizes) == 1
+            loaded_shard_id = self.shard_ids[0]
+        i = self.shard_ids.index(loaded_shard_id)
+        dst = param.data.narrow(0, sum(self.output_sizes[:i]), self.output_sizes[i])
+        assert dst.shape == loaded_weight.shape, f"shard {loaded_shard_id!r}: {tuple(loaded_weight.shape)} does not fit {tuple(dst.shape)}"
+        dst.copy_(loaded_weight)
+
+    def split(self, y: torch.Tensor):
+        return y.split(self.output_sizes, dim=-1)
+
+    def forward(self, x: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
+        return ops.linear_any(x, self.weight.data, None, out_f32)

@@ -44,3 +44,30 @@ def get_rope(head_size: int, rotary_dim: int, max_position: int, base: float, ro
         kind = rope_scaling.get("rope_type", "default")
         assert kind == "default", f"rope_type '{kind}' is not supported"
     return _cached_rope(head_size, rotary_dim, max_position, float(base))
+
+
+def rotary_frequencies(dims: int, base: float, yarn: dict | None = None) -> tuple[torch.Tensor, float]:
+    """(fp32 frequencies of the dims/2 rotation pairs, factor on cos and sin) for kernels that form the angle
+    position * frequency themselves (nvh_attn_rotary_prep), so no table bounds the position.
+
+    Without `yarn`: base^(-2i/dims) and 1.  With yarn = {factor, original, fast, slow} (YaRN: "Efficient Context Window
+    Extension of Large Language Models", Peng et al.): a pair that turns more than `fast` times over the `original`
+    context keeps its frequency, one that turns fewer than `slow` times is divided by `factor`, pairs in between blend
+    linearly in the pair index; cos and sin are scaled by 0.1 ln(factor) + 1.  Computed in float64 on the host."""
+    import math
+    half = dims // 2
+    freq = [base ** (-2.0 * i / dims) for i in range(half)]
+    if not yarn:
+        return torch.tensor(freq, dtype=torch.float64).float(), 1.0
+    factor, original = float(yarn["factor"]), float(yarn["original"])
+
+    def pair_index(turns: float) -> float:         # the (fractional) pair that makes `turns` turns over the original context
+        return dims * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+    lo = max(math.floor(pair_index(float(yarn["fast"]))), 0)
+    hi = min(math.ceil(pair_index(float(yarn["slow"]))), dims - 1)
+    out = []
+    for i, f in enumerate(freq):
+        ramp = min(max((i - lo) / max(hi - lo, 0.001), 0.0), 1.0)
+        out.append(f / factor * ramp + f * (1.0 - ramp))
+    return torch.tensor(out, dtype=torch.float64).float(), 0.1 * math.log(factor) + 1.0

@@ -553,3 +553,173 @@ def sample_with_noise(logits: torch.Tensor, temperatures: torch.Tensor, noise: t
     _hip.call("nvh_sample_with_noise", logits.data_ptr(), f, logits.stride(0), temperatures.data_ptr(), noise.data_ptr(),
               out.data_ptr(), logits.shape[0], logits.shape[1], _p(ws), _stream())
     return out
+
+
+# ---------------------------------------------------------------- fp32 residual stream, free head sizes, bf16 or fp32 activations
+F32 = torch.float32
+
+
+def _act_flag(*tensors) -> int:
+    """0 for bf16 activations, 1 for fp32; every tensor must be on the GPU and of the one type."""
+    dt = tensors[0].dtype
+    for t in tensors:
+        if not t.is_cuda or t.dtype != dt:
+            raise TypeError(f"expected GPU tensors of one activation type, got {t.dtype} on {t.device} beside {dt}")
+    if dt not in (BF16, F32):
+        raise TypeError(f"activation type {dt} unsupported (bf16 or fp32)")
+    return int(dt == F32)
+
+
+def linear_any(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None = None, out_f32: bool = False) -> torch.Tensor:
+    """y = x @ W^T (+ bias) for any sizes: bf16 shapes the tuned GEMM takes (K % 64 == 0, N % 4 == 0, 16-byte rows) go
+    there, everything else - ragged sizes, fp32 operands, an fp32 result of bf16 operands - to the any-shape kernel.  The
+    route depends on (N, K) and the types only, never on the number of rows."""
+    f = _act_flag(x, weight)
+    k, n = x.shape[-1], weight.shape[0]
+    assert weight.is_contiguous() and weight.shape[1] == k and x.stride(-1) == 1
+    x2 = x.reshape(-1, k)
+    m = x2.shape[0]
+    if not f and not out_f32 and k % 64 == 0 and n % 4 == 0 and x2.stride(0) % 8 == 0 and x2.data_ptr() % 16 == 0:
+        y = torch.empty(m, n, dtype=BF16, device=x.device)
+        if m:
+            _hip.call("nvh_gemm_bf16_nt", x2.data_ptr(), x2.stride(0), weight.data_ptr(), _p(bias), y.data_ptr(), n, m, n, k, 1, 0, _stream())
+        return y
+    out_f32 = bool(out_f32 or f)
+    y = torch.empty(m, n, dtype=F32 if out_f32 else BF16, device=x.device)
+    _hip.call("nvh_gemm_any_nt", x2.data_ptr(), x2.stride(0), weight.data_ptr(), _p(bias), y.data_ptr(), n, m, n, k, f, int(out_f32), _stream())
+    return y
+
+
+def embedding_stream(ids: torch.Tensor, table: torch.Tensor, x0: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 rows table[ids]; `x0` (a view [T, dim] of the table's type, row stride free) receives the same rows."""
+    f = _act_flag(table)
+    assert ids.dtype == torch.int64 and table.is_contiguous()
+    t, dim = ids.numel(), table.shape[1]
+    x = torch.empty(t, dim, dtype=F32, device=table.device)
+    assert x0 is None or (x0.dtype == table.dtype and x0.shape == (t, dim) and x0.stride(1) == 1)
+    _hip.call("nvh_embedding_stream", ids.data_ptr(), table.data_ptr(), x.data_ptr(), _p(x0), x0.stride(0) if x0 is not None else 0,
+              t, dim, table.shape[0], f, _stream())
+    return x
+
+
+def residual_dyt(x: torch.Tensor, y: torch.Tensor | None = None, post=None, bias: torch.Tensor | None = None, accumulate: bool = True,
+                 nxt=None, out: torch.Tensor | None = None) -> torch.Tensor | None:
+    """x <- (x if accumulate else 0) + post(y) + bias in place (fp32 rows); returns next(x) in the activation type, or None
+    without `nxt`.  post / nxt are (alpha, weight, bias) triples of a Dynamic-Tanh norm."""
+    assert x.dtype == F32 and x.is_contiguous() and x.dim() == 2
+    rows, dim = x.shape
+    ref = nxt[1] if nxt is not None else (post[1] if post is not None else (y if y is not None else bias))
+    f = _act_flag(ref)
+    h = None
+    if nxt is not None:
+        h = out if out is not None else torch.empty(rows, dim, dtype=ref.dtype, device=x.device)
+        assert h.stride(1) == 1 and h.shape == (rows, dim)
+    assert y is None or (y.shape == (rows, dim) and y.stride(1) == 1 and y.dtype == ref.dtype)
+    pa, pw, pb = post if post is not None else (None, None, None)
+    na, nw, nb = nxt if nxt is not None else (None, None, None)
+    _hip.call("nvh_residual_dyt", _p(y), y.stride(0) if y is not None else 0, _p(pa), _p(pw), _p(pb), _p(bias), x.data_ptr(), int(accumulate),
+              _p(na), _p(nw), _p(nb), _p(h), h.stride(0) if h is not None else 0, rows, dim, f, _stream())
+    return h
+
+
+def stream_cast_(x: torch.Tensor, out: torch.Tensor) -> None:
+    """out[:, :dim] = x in out's type (out may be wider: its other columns stay)."""
+    f = _act_flag(out)
+    assert x.dtype == F32 and x.is_contiguous() and out.stride(1) == 1 and out.shape[0] == x.shape[0] and out.shape[1] >= x.shape[1]
+    _hip.call("nvh_stream_cast", x.data_ptr(), out.data_ptr(), out.stride(0), x.shape[0], x.shape[1], f, _stream())
+
+
+def gelu_tanh_mul(gate_up: torch.Tensor) -> torch.Tensor:
+    f = _act_flag(gate_up)
+    assert gate_up.dim() == 2 and gate_up.stride(1) == 1
+    rows, inter = gate_up.shape[0], gate_up.shape[1] // 2
+    y = torch.empty(rows, inter, dtype=gate_up.dtype, device=gate_up.device)
+    _hip.call("nvh_gelu_tanh_mul", gate_up.data_ptr(), gate_up.stride(0), y.data_ptr(), rows, inter, f, _stream())
+    return y
+
+
+def gather_rows_f32(x: torch.Tensor, index: torch.Tensor) -> torch.Tensor:
+    assert x.dtype == F32 and x.is_contiguous() and index.dtype == torch.int32 and x.is_cuda and index.is_cuda
+    out = torch.empty(index.numel(), x.shape[1], dtype=F32, device=x.device)
+    if index.numel() == 0:
+        return out
+    _hip.call("nvh_gather_rows_f32", x.data_ptr(), index.data_ptr(), out.data_ptr(), index.numel(), x.shape[1], _stream())
+    return out
+
+
+def logit_softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """fp32 cap * tanh(logits / cap); cap <= 0: the logits in fp32."""
+    f = _act_flag(logits)
+    assert logits.dim() == 2 and logits.stride(1) == 1
+    out = torch.empty(logits.shape, dtype=F32, device=logits.device)
+    _hip.call("nvh_logit_softcap", logits.data_ptr(), logits.stride(0), out.data_ptr(), logits.shape[0], logits.shape[1], float(cap or 0.0), f, _stream())
+    return out
+
+
+def attn_rotary_prep(proj, q_norm, k_norm, eps: float, positions, qk_freq, qk_mag: float, rot_dims: int, v_freq, k_cache, v_cache,
+                     slot_mapping, heads: int, kv_heads: int, dim: int, vdim: int, gated: bool = True, qk_interleaved: bool = False,
+                     v_interleaved: bool = False):
+    """(q [T, H*dim], sigmoid gate fp32 [T, H] | None) from the fused projection rows [q | k | v | gate]; k and v go to their
+    cache rows (see nvh_attn_rotary_prep)."""
+    f = _act_flag(proj, q_norm, k_norm, k_cache, v_cache)
+    t = proj.shape[0]
+    assert proj.stride(1) == 1 and positions.dtype == torch.int64 and slot_mapping.dtype == torch.int32 and slot_mapping.numel() == t
+    assert qk_freq is None or (qk_freq.dtype == F32 and qk_freq.numel() * 2 == rot_dims)
+    assert v_freq is None or (v_freq.dtype == F32 and v_freq.numel() * 2 == vdim)
+    assert q_norm.numel() == heads * dim and k_norm.numel() == kv_heads * dim and k_cache.is_contiguous() and v_cache.is_contiguous()
+    q = torch.empty(t, heads * dim, dtype=proj.dtype, device=proj.device)
+    gate = torch.empty(t, heads, dtype=F32, device=proj.device) if gated else None
+    _hip.call("nvh_attn_rotary_prep", proj.data_ptr(), proj.stride(0), q_norm.data_ptr(), k_norm.data_ptr(), float(eps), positions.data_ptr(),
+              _p(qk_freq), float(qk_mag), rot_dims, int(qk_interleaved), _p(v_freq), int(v_interleaved), q.data_ptr(), _p(gate),
+              k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(), t, heads, kv_heads, dim, vdim, f, _stream())
+    return q, gate
+
+
+def attn_paged_any(q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, scale: float, heads: int, kv_heads: int, dim: int,
+                   vdim: int, gate=None, v_freq=None, v_interleaved: bool = False) -> torch.Tensor:
+    """Causal attention of the packed queries q [T, H*dim] over paged caches [pages, page, G, dim|vdim]; out [T, H*vdim]."""
+    f = _act_flag(q, k_cache, v_cache)
+    t = q.shape[0]
+    batch = context_lens.numel()
+    assert q.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
+    assert context_lens.dtype == torch.int32 and block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
+    assert cu_seqlens_q is None or (cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.numel() == batch + 1)
+    assert cu_seqlens_q is not None or t == batch
+    assert gate is None or (gate.dtype == F32 and gate.shape == (t, heads) and gate.is_contiguous())
+    out = torch.empty(t, heads * vdim, dtype=q.dtype, device=q.device)
+    _hip.call("nvh_attn_paged_any", q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(),
+              block_tables.data_ptr(), block_tables.stride(0), batch, t, k_cache.shape[1], heads, kv_heads, dim, vdim, float(scale),
+              _p(gate), _p(v_freq), int(v_interleaved), out.data_ptr(), f, _stream())
+    return out
+
+
+def delta_rule(r, k, v, a_raw, lowrank, w2, w0, a_bias, state, slots, cu_seqlens_q, context_lens, heads: int, dk: int,
+               decay_scale: float) -> torch.Tensor:
+    """One step of the generalized delta rule over the packed tokens: fp32 outputs [T, H*dk]; `state` [slots, H, dk, dk] fp32 is
+    read (unless the sequence starts in this step) and left updated.  r, k, v, a_raw, lowrank: column views of the fused
+    projection output (row stride free)."""
+    f = _act_flag(r, k, v, a_raw, lowrank, w2, w0, a_bias)
+    t = r.shape[0]
+    batch = context_lens.numel()
+    for x in (r, k, v, a_raw, lowrank):
+        assert x.stride(1) == 1 and x.shape[0] == t
+    assert state.dtype == F32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dk, dk) and slots.dtype == torch.int32
+    assert w2.is_contiguous() and w2.shape[0] == heads * dk and (cu_seqlens_q is None or cu_seqlens_q.dtype == torch.int32)
+    rank = w2.shape[1]
+    wua = torch.empty(t, 3, heads * dk, dtype=F32, device=r.device)
+    _hip.call("nvh_delta_prep", k.data_ptr(), k.stride(0), a_raw.data_ptr(), a_raw.stride(0), lowrank.data_ptr(), lowrank.stride(0),
+              w2.data_ptr(), w0.data_ptr(), a_bias.data_ptr(), wua.data_ptr(), t, heads, dk, rank, float(decay_scale), f, _stream())
+    out = torch.empty(t, heads * dk, dtype=F32, device=r.device)
+    _hip.call("nvh_delta_scan", r.data_ptr(), r.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), wua.data_ptr(),
+              state.data_ptr(), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(), out.data_ptr(), batch, heads, dk, dk, f, _stream())
+    return out
+
+
+def delta_post(o: torch.Tensor, norm_weight: torch.Tensor, gate: torch.Tensor | None, heads: int, dv: int, eps: float) -> torch.Tensor:
+    """o / rms_head(o) * norm_weight * sigmoid(gate) in norm_weight's type; gate: a column view of the projection output."""
+    f = _act_flag(norm_weight) if gate is None else _act_flag(norm_weight, gate)
+    assert o.dtype == F32 and o.is_contiguous() and o.shape[1] == heads * dv and (gate is None or gate.stride(1) == 1)
+    y = torch.empty(o.shape, dtype=norm_weight.dtype, device=o.device)
+    _hip.call("nvh_delta_post", o.data_ptr(), norm_weight.data_ptr(), _p(gate), gate.stride(0) if gate is not None else 0, y.data_ptr(),
+              y.stride(0), o.shape[0], heads, dv, float(eps), f, _stream())
+    return y

@@ -9,5 +9,6 @@ class SamplingParams:
     ignore_eos: bool = False
 
     def __post_init__(self):
-        # the sampler always races against exponential noise; temperature 0 is undefined for it
-        assert self.temperature > 1e-10, "greedy sampling is not permitted"
+        # temperature 0 selects the most likely token (the sampler's race runs without noise for such a row; the
+        # reference forbids it); anything between 0 and 1e-10 would overflow logits / T
+        assert self.temperature == 0 or self.temperature > 1e-10, "temperature must be 0 (greedy) or above 1e-10"

@@ -1,7 +1,7 @@
 """Per-step attention metadata shared between the runner and the operator modules.
 
-Mirrors nanovllm/utils/context.py:22-111 of the reference (same eight fields, same
-positional order in set_context) so callers and operator modules written against
+Mirrors nanovllm/utils/context.py:22-111 of the reference (its eight fields in the same
+positional order in set_context, then the state slots of recurrent layers) so callers and operator modules written against
 the reference keep working.  One record per process, replaced every step.
 """
 from __future__ import annotations
@@ -11,7 +11,7 @@ from dataclasses import dataclass
 import torch
 
 FIELDS = ("cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k", "slot_mapping", "context_lens",
-          "block_tables", "seq_need_compute_logits")
+          "block_tables", "seq_need_compute_logits", "state_slots")
 
 
 @dataclass
@@ -24,6 +24,7 @@ class Context:
     context_lens: torch.Tensor | None = None      # int32 [B]
     block_tables: torch.Tensor | None = None      # int32 [B, W], -1 padded (0 padded in graph buffers)
     seq_need_compute_logits: torch.Tensor | None = None   # int32 [B']
+    state_slots: torch.Tensor | None = None       # int32 [B]: recurrent-state slot of every sequence (-1: a padded row); not in the reference
 
 
 _current = Context()
@@ -35,10 +36,10 @@ def get_context() -> Context:
 
 def set_context(*args, **kwargs) -> None:
     """set_context(cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, slot_mapping,
-    context_lens, block_tables, seq_need_compute_logits); every argument optional."""
+    context_lens, block_tables, seq_need_compute_logits[, state_slots]); every argument optional."""
     global _current
     if len(args) > len(FIELDS):
-        raise TypeError("set_context takes at most 8 positional arguments")
+        raise TypeError(f"set_context takes at most {len(FIELDS)} positional arguments")
     values = dict(zip(FIELDS, args))
     for key, val in kwargs.items():
         if key not in FIELDS or key in values:

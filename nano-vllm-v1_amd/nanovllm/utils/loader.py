@@ -31,8 +31,29 @@ def load_tensors(model: nn.Module, named_tensors, loaded: set | None = None) -> 
     ``loaded`` collects the parameter names that received data."""
     packed = getattr(model, "packed_modules_mapping", {})
     params = dict(model.named_parameters())
+    target_of = getattr(model, "weight_target", None)      # a model that names its checkpoint tensors its own way
     n = 0
     for name, tensor in named_tensors:
+        if target_of is not None:
+            pname, shard_id = target_of(name)
+            if pname not in params:
+                raise KeyError(f"checkpoint tensor {name!r} maps to {pname!r}, which is not a parameter of the model")
+            param = params[pname]
+            loader = getattr(param, "weight_loader", None)
+            if shard_id is not None:
+                loader(param, tensor, shard_id)
+                if loaded is not None:
+                    loaded.add((pname, shard_id))
+            elif loader is not None:
+                loader(param, tensor)
+            else:
+                if tuple(param.shape) != tuple(tensor.shape):
+                    raise ValueError(f"checkpoint tensor {name!r} has shape {tuple(tensor.shape)}, parameter {pname!r} {tuple(param.shape)}")
+                default_weight_loader(param, tensor)
+            if loaded is not None:
+                loaded.add(pname)
+            n += 1
+            continue
         for key, (target, shard_id) in packed.items():
             if key in name:
                 pname = name.replace(key, target)
@@ -63,6 +84,12 @@ def check_all_loaded(model: nn.Module, loaded: set) -> None:
     for target, shard_id in packed.values():
         shards_of.setdefault(target, set()).add(shard_id)
     incomplete = []
+    for name, p in model.named_parameters():                # merged parameters that list their shards themselves
+        ids = getattr(p, "shard_ids", None)
+        if ids and len(ids) > 1 and name in loaded:
+            lacking = sorted(str(i) for i in ids if (name, i) not in loaded)
+            if lacking:
+                incomplete.append(f"{name} (shards {', '.join(lacking)} missing)")
     for name in sorted(n for n in loaded if isinstance(n, str)):
         for target, ids in shards_of.items():
             if f".{target}." in f".{name}" or name.startswith(target + "."):
@@ -88,6 +115,17 @@ def load_model(model: nn.Module, path: str) -> int:
             n += load_tensors(model, ((name, f.get_tensor(name)) for name in f.keys()), loaded)
     check_all_loaded(model, loaded)
     return n
+
+
+def checkpoint_shapes(path: str) -> dict:
+    """Tensor name -> shape over every safetensors file of a model directory (headers only: no data is read)."""
+    from safetensors import safe_open
+    shapes = {}
+    for file in sorted(glob(os.path.join(path, "*.safetensors"))):
+        with safe_open(file, "pt", "cpu") as f:
+            for name in f.keys():
+                shapes[name] = tuple(f.get_slice(name).get_shape())
+    return shapes
 
 
 def has_checkpoint(path: str) -> bool:
