@@ -714,12 +714,12 @@ class ModelRunner:
         reset_context()
         return out
 
-    @torch.inference_mode()
     def _logits_of_rows(self, rows):
         if hasattr(self.model, "compute_logits_rows"):
             return self.model.compute_logits_rows(rows)
         return self.model.lm_head.forward_rows(rows)
 
+    @torch.inference_mode()
     def forward_logits(self, seqs, gather=True, rows=None):
         """Everything of a step up to the sampler: (logits [B', V] | None, temperatures | None, need)
         with ``need`` a HOST int32 tensor (indices into ``seqs`` of the rows of ``logits``).  logits is
