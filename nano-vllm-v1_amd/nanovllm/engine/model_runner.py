@@ -226,7 +226,6 @@ class ModelRunner:
         config.recurrent_state = bool(getattr(cls, "has_recurrent_state", False))
         if self.generic:
             assert self.world_size == 1, f"{cls.__name__} is served on one GPU (its layers are not tensor-parallel)"
-            self.enforce_eager = True            # its steps are launched one by one (no captured decode graph yet)
         prev_dtype = torch.get_default_dtype()
         torch.set_default_dtype(dtype)
         torch.set_default_device(self.device)
@@ -550,6 +549,8 @@ class ModelRunner:
         """Key-range count of the decode attention for a batch of `bs`: chosen per graph bucket and for the longest
         context a sequence may reach, so a captured graph and an eager step of the same batch sum in the same
         order (enforce_eager does not change a single bit of the output)."""
+        if self.generic:
+            return 1                            # (its attention kernel takes no key-range split)
         bucket = next((b for b in self.decode_buckets() if b >= bs), bs)
         hkv = self.model.model.layers[0].self_attn.num_kv_heads
         return ops.suggest_decode_splits(bucket, hkv, self.config.max_model_len)
@@ -576,7 +577,7 @@ class ModelRunner:
         sequences with a long context among them are offered 16 ranges of at least 512 keys (short ones still use
         one); larger batches keep the uniform split, where that many idle workgroups would cost more than they save."""
         short = self.decode_splits(bs)
-        if max_context <= self.LONG_CONTEXT or short >= 16 or bs > 64:
+        if self.generic or max_context <= self.LONG_CONTEXT or short >= 16 or bs > 64:
             return short, 0
         return 16, 512
 
@@ -857,7 +858,8 @@ class _DecodeGraph:
         self.items_cap = bs + runner.ITEM_SLACK
         sizes = dict(input_ids=bs * 8, positions=bs * 8, slot_mapping=bs * 4, context_lens=bs * 4,
                      block_tables=bs * width * 4, temperatures=bs * 4, item_seq=self.items_cap * 4,
-                     item_range=self.items_cap * 4, seq_active=bs * 4, seq_chunk=bs * 4, fed_dst=bs * 4, fed_src=bs * 4)
+                     item_range=self.items_cap * 4, seq_active=bs * 4, seq_chunk=bs * 4, fed_dst=bs * 4, fed_src=bs * 4,
+                     state_slots=bs * 4)
         self.offs, n = {}, 0
         for name, nbytes in sizes.items():
             self.offs[name] = (n, nbytes)
@@ -869,9 +871,11 @@ class _DecodeGraph:
         self.h = {k: v.numpy() for k, v in hv.items()}
         self.d = dv
         self.h["slot_mapping"][:] = -1
+        self.h["state_slots"][:] = -1                                 # padding rows own no state: the recurrent kernels skip them
         self._plan_items()
         self.dev.copy_(self.host)
-        set_context(slot_mapping=dv["slot_mapping"], context_lens=dv["context_lens"], block_tables=dv["block_tables"])
+        set_context(slot_mapping=dv["slot_mapping"], context_lens=dv["context_lens"], block_tables=dv["block_tables"],
+                    state_slots=dv["state_slots"] if runner.config.recurrent_state else None)
         self.splits = runner.decode_splits(bs)                        # batches without a long context
         has_long = runner.native is not None and runner.decode_plan(bs, 1 << 30)[1]
         self.graph_long = self.out_long = None
@@ -918,7 +922,8 @@ class _DecodeGraph:
                     block_tables=v("block_tables", torch.int32, bs, w), temperatures=v("temperatures", torch.float32, bs),
                     item_seq=v("item_seq", torch.int32, self.items_cap), item_range=v("item_range", torch.int32, self.items_cap),
                     seq_active=v("seq_active", torch.int32, bs), seq_chunk=v("seq_chunk", torch.int32, bs),
-                    fed_dst=v("fed_dst", torch.int32, bs), fed_src=v("fed_src", torch.int32, bs))
+                    fed_dst=v("fed_dst", torch.int32, bs), fed_src=v("fed_src", torch.int32, bs),
+                    state_slots=v("state_slots", torch.int32, bs))
 
     def replay(self, fb, seqs, want_temps: bool, prev_sampled=None):
         n = len(seqs)
@@ -931,6 +936,9 @@ class _DecodeGraph:
         h["slot_mapping"][n:] = -1
         h["context_lens"][:n] = fb["context_lens"]
         h["context_lens"][n:] = 0
+        if self.runner.config.recurrent_state:
+            h["state_slots"][:n] = np.fromiter((s.state_slot for s in seqs), dtype=np.int32, count=n)
+            h["state_slots"][n:] = -1
         tb = fb["block_tables"]
         h["block_tables"][:n, :tb.shape[1]] = tb
         if want_temps:

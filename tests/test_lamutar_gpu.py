@@ -388,6 +388,7 @@ def test_greedy_generation_through_the_engine(loop_case):
     llm = LLM(loop_case.path, dtype="float32", max_num_seqs=4, max_num_batched_tokens=32, max_model_len=128, num_kvcache_blocks=6,
               chunked_prefill=True)
     try:
+        assert llm.model_runner.graphs, "one-token steps are expected to replay captured graphs"
         outs = llm.generate(prompts, SamplingParams(temperature=0.0, max_tokens=12, ignore_eos=True), use_tqdm=False)
     finally:
         llm.exit()
@@ -396,3 +397,21 @@ def test_greedy_generation_through_the_engine(loop_case):
         for _ in range(12):
             toks.append(int(R.forward(CFG_LOOP, loop_case.W, toks)[-1].argmax()))
         assert out["token_ids"] == toks[len(prompt):]
+
+
+def test_temperature_zero_rows_take_the_maximum():
+    """Rows with temperature 0 beside sampled rows in one sampler call: the greedy rows are the row maxima (lowest index
+    among equals), whatever the seed."""
+    from nanovllm import ops
+    g = torch.Generator().manual_seed(3)
+    logits = torch.randn(6, 1000, generator=g)
+    logits[2, 17] = logits[2, 500] = 9.0                      # a tie: the lower index wins
+    temps = torch.tensor([0.0, 1.0, 0.0, 0.7, 0.0, 0.0])
+    for dtype in (torch.float32, torch.bfloat16):
+        lg = logits.to(dtype).cuda()
+        for seed in (1, 2):
+            ids = ops.sample(lg, temps.cuda(), seed, 5).cpu()
+            want = lg.float().cpu().argmax(-1)
+            for r in (0, 4, 5):
+                assert ids[r] == want[r]
+            assert ids[2] == 17
