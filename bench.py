@@ -101,14 +101,21 @@ class Driver:
         self.Sequence = Sequence
         self.runner = runner
         self.next_page = 0
+        self.next_slot = 0
         self.num_pages = runner.config.num_kvcache_blocks
 
     def reset(self):
         self.next_page = 0
+        self.next_slot = 0
 
     def new_seq(self, tokens, temperature=0.6):
         from nanovllm.sampling_params import SamplingParams
-        return self.Sequence(tokens, SamplingParams(temperature=temperature, max_tokens=1 << 30, ignore_eos=True))
+        s = self.Sequence(tokens, SamplingParams(temperature=temperature, max_tokens=1 << 30, ignore_eos=True))
+        if getattr(self.runner.config, "recurrent_state", False):     # models with a per-sequence state: one slot each
+            s.state_slot = self.next_slot
+            self.next_slot += 1
+            assert self.next_slot <= self.runner.config.num_state_slots, "state slots exhausted"
+        return s
 
     def grow(self, s, ctx):
         while len(s.block_table) * PAGE < ctx:
@@ -450,8 +457,75 @@ def cpu_baseline(hf):
                 host_cpus=os.cpu_count())
 
 
+HYBRID_SIZES = {
+    # layer sizes of two public dense models, eight layers each (enough to time a layer; equal in both designs)
+    "w1024": dict(width=1024, heads=16, kv_heads=8, head_dim=128, ff=3072, layers=8, vocab=32768),
+    "w2048": dict(width=2048, heads=16, kv_heads=8, head_dim=128, ff=6144, layers=8, vocab=32768),
+}
+
+
+def hybrid_compare(args):
+    """--hybrid-compare: prefill and decode throughput of the Lamutar design (attention and delta-rule layers 1:2, fp32 residual
+    stream, operator modules + captured decode graphs) beside Qwen3 (the closest model the engine serves: native executor)
+    at equal width, heads, feed-forward size, depth and vocabulary; random weights, bf16.  One JSON line."""
+    import tempfile
+    from nanovllm.config import Config
+    from nanovllm.engine.model_runner import ModelRunner
+
+    def lamutar_cfg(z):
+        attn = {"type": "attention", "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["head_dim"], "vdim": z["head_dim"],
+                                               "scale": z["head_dim"] ** -0.5,
+                                               "rot": {"base": 1e6, "dims": z["head_dim"] // 2, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
+                "mlp": {"kind": "dense", "ff": z["ff"]}}
+        delta = {"type": "general_delta", "mixer": {"heads": z["width"] // 64, "dim": 64}, "mlp": {"kind": "dense", "ff": z["ff"]}}
+        return {"architecture": "Lamutar", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "loop": None,
+                "layers": [attn if i % 3 == 0 else delta for i in range(z["layers"])]}
+
+    def qwen3_cfg(z):
+        return {"architectures": ["Qwen3ForCausalLM"], "hidden_size": z["width"], "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
+                "num_key_value_heads": z["kv_heads"], "head_dim": z["head_dim"], "intermediate_size": z["ff"], "vocab_size": z["vocab"],
+                "max_position_embeddings": 40960, "rms_norm_eps": 1e-6, "rope_theta": 1000000, "tie_word_embeddings": False, "hidden_act": "silu",
+                "attention_bias": False, "torch_dtype": "bfloat16"}
+
+    b, ctx, chunk = args.batch if args.batch != 256 else 64, args.context, 1024
+    results = {}
+    for name in (args.hybrid_sizes.split(",") if args.hybrid_sizes else HYBRID_SIZES):
+        z = HYBRID_SIZES[name]
+        results[name] = {}
+        for design, make in (("lamutar", lamutar_cfg), ("qwen3", qwen3_cfg)):
+            with tempfile.TemporaryDirectory() as d:
+                with open(os.path.join(d, "config.json"), "w") as f:
+                    json.dump(make(z), f)
+                steps = args.steps + args.warmup
+                pages = b * ((ctx + steps + PAGE) // PAGE + 2) + 8
+                cfg = Config(d, max_num_batched_tokens=chunk, max_num_seqs=b, max_model_len=ctx + steps + 2 * PAGE, chunked_prefill=True,
+                             num_kvcache_blocks=pages)
+                runner = ModelRunner(cfg, 0, [])
+            driver = Driver(runner)
+            g = torch.Generator().manual_seed(0)
+            seqs = [driver.new_seq(torch.randint(0, z["vocab"], (ctx,), generator=g).tolist()) for _ in range(b)]
+            ptimes = driver.prefill(seqs, chunk)                          # synchronous: one chunk timed at a time
+            steady = sorted(x[0] for x in ptimes[len(ptimes) // 4:])
+            chunk_s = steady[len(steady) // 2]
+            dt = time_decode(driver, seqs, args.steps, args.warmup, False)
+            results[name][design] = dict(prefill_tok_s=round(min(chunk, ctx) / chunk_s, 1), prefill_ms_per_chunk=round(chunk_s * 1e3, 3),
+                                         decode_tok_s=round(b * args.steps / dt, 1), decode_ms_per_step=round(dt / args.steps * 1e3, 4),
+                                         graphs=bool(runner.graphs))
+            runner.exit()
+            del runner, driver, seqs
+            torch.cuda.empty_cache()
+        lam, q = results[name]["lamutar"], results[name]["qwen3"]
+        results[name]["lamutar_over_qwen3"] = dict(prefill=round(lam["prefill_tok_s"] / q["prefill_tok_s"], 3),
+                                                   decode=round(lam["decode_tok_s"] / q["decode_tok_s"], 3))
+    print(json.dumps(dict(metric="prefill and decode tok/s, Lamutar beside Qwen3 at equal layer sizes (bf16, random weights)",
+                          batch=b, context=ctx, chunk_tokens=chunk, steps=args.steps, warmup=args.warmup, sizes=results)))
+
+
 def main():
     ap = argparse.ArgumentParser()
+    ap.add_argument("--hybrid-compare", action="store_true",
+                    help="instead of the headline workload: the Lamutar design beside Qwen3 at equal layer sizes (see hybrid_compare)")
+    ap.add_argument("--hybrid-sizes", default="", help="comma-separated subset of " + ",".join(HYBRID_SIZES))
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
@@ -460,6 +534,9 @@ def main():
     ap.add_argument("--no-extras", action="store_true", help="skip sweeps, long prefill and the CPU baseline")
     ap.add_argument("--model", default="qwen3-0.6b", help="directory name under nano-vllm-v1_amd/model_configs (default: the headline model)")
     args = ap.parse_args()
+    if args.hybrid_compare:
+        torch.cuda.set_device(0)
+        return hybrid_compare(args)
 
     world = int(os.environ.get("WORLD_SIZE", "1"))
     rank = int(os.environ.get("RANK", "0"))

@@ -538,19 +538,18 @@ int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const void* v_cac
                            int32_t act_f32, nvh_stream_t stream);
 
 /* Generalized delta rule, state [slots, H, dk, dv] fp32:  S <- diag(w) S - (a u)(u^T S) + k v^T,  o = S^T r.
- * nvh_delta_prep: out fp32 [T, 3, H dk] = w | u | a u with w = exp(-decay_scale sigmoid(w0 + w2 tanh(lowrank))),
- * a = sigmoid(a_raw + a_bias), u = k / sqrt(sum_head k^2 + 1e-6).
+ * nvh_delta_prep: out fp32 [T, H, 6, dk] = r | k | w | u | a u | v per head, with w = exp(-decay_scale sigmoid(w0 + w2 tanh(lowrank))),
+ * a = sigmoid(a_raw + a_bias), u = k / sqrt(sum_head k^2 + 1e-6) (value size = key size dk).
  * nvh_delta_scan: sequence b owns state slot slots[b] (< 0: a padded row) and this step's tokens cu_seqlens_q[b] ..
  * (NULL: row b); it starts from zero when context_lens[b] equals its token count, else from the slot, and leaves the
- * state there; out fp32 [T, H dv].  dk % 4 == 0, dk <= 256.
+ * state there; out fp32 [T, H dk].  dk % 4 == 0, dk <= 256.
  * nvh_delta_post: y (type A) = o / rms_head(o) * norm_weight * sigmoid(gate) (gate NULL: none). */
-int32_t nvh_delta_prep(const void* k, int64_t k_stride, const void* a_raw, int64_t a_stride, const void* lowrank, int64_t lowrank_stride,
+int32_t nvh_delta_prep(const void* r, int64_t r_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                       const void* a_raw, int64_t a_stride, const void* lowrank, int64_t lowrank_stride,
                        const void* w2, const void* w0, const void* a_bias, float* out, int64_t num_tokens, int64_t heads, int64_t dk,
                        int64_t rank, float decay_scale, int32_t act_f32, nvh_stream_t stream);
-int32_t nvh_delta_scan(const void* r, int64_t r_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
-                       const float* wua, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
-                       const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
-                       int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_delta_scan(const float* pack, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                       const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, nvh_stream_t stream);
 int32_t nvh_delta_post(const float* o, const void* norm_weight, const void* gate, int64_t gate_stride, void* y, int64_t y_stride,
                        int64_t rows, int64_t heads, int64_t dv, float eps, int32_t act_f32, nvh_stream_t stream);
 

@@ -3,11 +3,12 @@
 // with a decay w in (0, 1) and a removal rate a per key channel and u the unit-length key.
 //   nvh_delta_prep   per token and channel, all in fp32: the decay from its low-rank logit
 //                    w = exp(-c * sigmoid(w0 + W2 tanh(l))) (c = e^-1/2 by default), a = sigmoid(a_raw + a_bias),
-//                    u = k / sqrt(sum k^2 + 1e-6); leaves [w | u | a*u] per token.
+//                    u = k / sqrt(sum k^2 + 1e-6); leaves, per token and head, the contiguous fp32 row
+//                    [r | k | w | u | a*u | v] that the scan reads.
 //   nvh_delta_scan   walks a sequence's tokens in order from the state its slot holds (or from zero when the sequence
 //                    starts) and leaves the state there.  Columns of S are independent of each other, so the work is
-//                    spread over (sequence, head, column); each column is held by four lanes (rows i mod 4), which
-//                    meet twice per token in a quad sum.  The order of every sum is fixed by the sizes alone: decoding
+//                    spread over (sequence, head, column); each column is held by 16 lanes (4 when dk is no multiple
+//                    of 16), each with every 16th (4th) row, which meet twice per token in a cross-lane sum.  The order of every sum is fixed by the sizes alone: decoding
 //                    token by token, in portions or in one piece gives the same bits.
 //   nvh_delta_post   per head: o / rms(o), times the norm weight and the sigmoid output gate, to the activation type.
 #include "common.h"
@@ -21,14 +22,14 @@ __device__ __forceinline__ float ldf(const A* p, int64_t i) {
 __device__ __forceinline__ float sigmoidf_(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 struct DeltaPrepArgs {
-    const void* k;             // [T, ld] rows of H*dk
-    int64_t k_stride;
+    const void *r, *k, *v;     // [T, ld] rows of H*dk
+    int64_t r_stride, k_stride, v_stride;
     const void* a_raw;         // [T, ld]
     int64_t a_stride;
     const void* lowrank;       // [T, ld] rows of `rank` (the first decay projection, before its tanh)
     int64_t l_stride;
     const void *w2, *w0, *a_bias;   // [H*dk, rank], [H*dk], [H*dk]
-    float* out;                // [T, 3, H*dk]: w | u | a*u
+    float* out;                // [T, H, 6, dk]: r | k | w | u | a*u | v per head, contiguous
     int H, dk, rank;
     float decay_scale;
 };
@@ -37,53 +38,58 @@ template <typename A>
 __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepArgs p) {
     extern __shared__ float tl[];                            // tanh of the low-rank row
     const int64_t t = blockIdx.x;
-    const int n = p.H * p.dk;
     for (int r = threadIdx.x; r < p.rank; r += 256) tl[r] = tanhf(ldf((const A*)p.lowrank, t * p.l_stride + r));
     __syncthreads();
-    float* out = p.out + t * 3 * n;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, dk = p.dk;
     for (int h = wave; h < p.H; h += 4) {
+        float* out = p.out + (t * p.H + h) * 6 * dk;
         float ss = 0.f;
-        for (int i = lane; i < p.dk; i += 64) {
-            const float kv = ldf((const A*)p.k, t * p.k_stride + h * p.dk + i);
+        for (int i = lane; i < dk; i += 64) {
+            const float kv = ldf((const A*)p.k, t * p.k_stride + h * dk + i);
             ss += kv * kv;
         }
         ss = wave_sum(ss);
         const float inv = 1.0f / sqrtf(ss + 1e-6f);
-        for (int i = lane; i < p.dk; i += 64) {
-            const int c = h * p.dk + i;
+        for (int i = lane; i < dk; i += 64) {
+            const int c = h * dk + i;
             float z = ldf((const A*)p.w0, c);
             const A* w2r = (const A*)p.w2 + (int64_t)c * p.rank;
             for (int r = 0; r < p.rank; ++r) z = __builtin_fmaf(ldf(w2r, r), tl[r], z);
-            const float u = ldf((const A*)p.k, t * p.k_stride + c) * inv;
+            const float kv = ldf((const A*)p.k, t * p.k_stride + c);
+            const float u = kv * inv;
             const float a = sigmoidf_(ldf((const A*)p.a_raw, t * p.a_stride + c) + ldf((const A*)p.a_bias, c));
-            out[c] = expf(-p.decay_scale * sigmoidf_(z));
-            out[n + c] = u;
-            out[2 * n + c] = a * u;
+            out[i] = ldf((const A*)p.r, t * p.r_stride + c);
+            out[dk + i] = kv;
+            out[2 * dk + i] = expf(-p.decay_scale * sigmoidf_(z));
+            out[3 * dk + i] = u;
+            out[4 * dk + i] = a * u;
+            out[5 * dk + i] = ldf((const A*)p.v, t * p.v_stride + c);
         }
     }
 }
 
 struct DeltaScanArgs {
-    const void *r, *k, *v;     // [T, stride] rows of H*dk (r, k) and H*dv (v)
-    int64_t r_stride, k_stride, v_stride;
-    const float* wua;          // [T, 3, H*dk]
-    float* state;              // [slots, H, dk, dv]
+    const float* pack;         // [T, H, 6, dk] from delta_prep_kernel
+    float* state;              // [slots, H, dk, dk]
     const int32_t* slots;      // [B]
     const int32_t* cu_seqlens_q;    // [B+1] or null (one token per sequence)
     const int32_t* context_lens;    // [B]: tokens of the sequence including this step's (a step that holds them all starts from zero)
-    float* out;                // [T, H*dv]
+    float* out;                // [T, H*dk]
     int H, dk, dv;
 };
 
-constexpr int DTOK = 8;        // tokens staged per round
-
-template <typename A, int DKQ>
+// Lanes per state column (SUBS: 16 when dk is a multiple of 16, else 4), rows i = SUBS * ii + sub held by lane `sub`; a
+// workgroup of 256 lanes owns 256 / SUBS columns of one (sequence, head).  Tokens are staged TOK at a time: the loads
+// of the next TOK tokens are in flight (in registers) while the current ones are walked from LDS.
+template <int DKQ, int SUBS>
 __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
-    extern __shared__ float sm[];                            // [DTOK][5 dk + dv]: r | k | w | u | au | v
+    constexpr int COLS = 256 / SUBS;
+    constexpr int CH = (5 * DKQ * SUBS + COLS + 255) / 256;  // loads per lane and token
+    constexpr int TOK = (32 / CH) < 2 ? 2 : (32 / CH);
+    extern __shared__ float sm[];                            // [TOK][5 dk + COLS]: r | k | w | u | au | v (this workgroup's columns)
     const int seq = blockIdx.x, head = blockIdx.y;
-    const int dk = p.dk, dv = p.dv, dkq = dk >> 2;
-    const int col = blockIdx.z * 64 + (threadIdx.x >> 2), sub = threadIdx.x & 3;
+    const int dk = p.dk, dv = p.dv, dkq = dk / SUBS;
+    const int col0 = blockIdx.z * COLS, lcol = threadIdx.x / SUBS, col = col0 + lcol, sub = threadIdx.x % SUBS;
     const bool live = col < dv;
     const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
     const int slot = p.slots[seq];
@@ -92,50 +98,74 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
     float* sp = p.state + (((int64_t)slot * p.H + head) * dk) * dv;
     float S[DKQ];
 #pragma unroll
-    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && ii < dkq) ? sp[(int64_t)(4 * ii + sub) * dv + col] : 0.f;
-    const int rowf = 5 * dk + dv, n = p.H * dk;
-    for (int t0 = lo; t0 < hi; t0 += DTOK) {
-        const int nt = min(DTOK, hi - t0);
-        __syncthreads();
-        for (int i = threadIdx.x; i < nt * rowf; i += 256) {
-            const int tt = i / rowf, e = i - tt * rowf;
-            const int64_t tok = t0 + tt;
-            float v;
-            if (e < dk) v = ldf((const A*)p.r, tok * p.r_stride + head * dk + e);
-            else if (e < 2 * dk) v = ldf((const A*)p.k, tok * p.k_stride + head * dk + e - dk);
-            else if (e < 5 * dk) v = p.wua[tok * 3 * n + (int64_t)((e - 2 * dk) / dk) * n + head * dk + (e - 2 * dk) % dk];
-            else v = ldf((const A*)p.v, tok * p.v_stride + head * dv + e - 5 * dk);
-            sm[i] = v;
+    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && ii < dkq) ? sp[(int64_t)(SUBS * ii + sub) * dv + col] : 0.f;
+    const int rowf = 5 * dk + COLS;
+    // Row of a token as this workgroup needs it: the five dk-vectors, then its COLS columns of v.  Every load is
+    // unconditional (indices clamped into the row and into the sequence), so all of a round's loads are in flight together.
+    float pre[TOK][CH];
+    const float* base = p.pack + (int64_t)head * 6 * dk;
+    const int64_t tok_stride = (int64_t)p.H * 6 * dk;
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int tt = 0; tt < TOK; ++tt) {
+            const int64_t tok = min(t0 + tt, hi - 1);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int e = threadIdx.x + 256 * c;
+                const int src = min(e < 5 * dk ? e : e + col0, 6 * dk - 1);
+                pre[tt][c] = base[tok * tok_stride + src];
+            }
         }
+    };
+    fetch(lo);
+    for (int t0 = lo; t0 < hi; t0 += TOK) {
+        const int nt = min(TOK, hi - t0);
+        __syncthreads();                                     // the previous round's readers are done
+#pragma unroll
+        for (int tt = 0; tt < TOK; ++tt)
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int e = threadIdx.x + 256 * c;
+                if (e < rowf) sm[tt * rowf + e] = pre[tt][c];
+            }
         __syncthreads();
+        if (t0 + TOK < hi) fetch(t0 + TOK);
         for (int tt = 0; tt < nt; ++tt) {
             const float* row = sm + tt * rowf;
             const float *rr = row, *kk = row + dk, *ww = row + 2 * dk, *uu = row + 3 * dk, *au = row + 4 * dk;
-            const float vj = live ? row[5 * dk + col] : 0.f;
+            const float vj = row[5 * dk + lcol];
             float dot = 0.f;
 #pragma unroll
             for (int ii = 0; ii < DKQ; ++ii)
-                if (ii < dkq) dot = __builtin_fmaf(uu[4 * ii + sub], S[ii], dot);
-            dot += NVH_DPP(dot, 0xB1);
-            dot += NVH_DPP(dot, 0x4E);
+                if (ii < dkq) dot = __builtin_fmaf(uu[SUBS * ii + sub], S[ii], dot);
+            if constexpr (SUBS == 16) {
+                dot = row16_sum(dot);
+            } else {
+                dot += NVH_DPP(dot, 0xB1);
+                dot += NVH_DPP(dot, 0x4E);
+            }
             float o = 0.f;
 #pragma unroll
             for (int ii = 0; ii < DKQ; ++ii)
                 if (ii < dkq) {
-                    const int i = 4 * ii + sub;
+                    const int i = SUBS * ii + sub;
                     const float s = __builtin_fmaf(ww[i], S[ii], __builtin_fmaf(kk[i], vj, -(au[i] * dot)));
                     S[ii] = s;
                     o = __builtin_fmaf(s, rr[i], o);
                 }
-            o += NVH_DPP(o, 0xB1);
-            o += NVH_DPP(o, 0x4E);
+            if constexpr (SUBS == 16) {
+                o = row16_sum(o);
+            } else {
+                o += NVH_DPP(o, 0xB1);
+                o += NVH_DPP(o, 0x4E);
+            }
             if (live && sub == 0) p.out[(int64_t)(t0 + tt) * p.H * dv + head * dv + col] = o;
         }
     }
     if (live) {
 #pragma unroll
         for (int ii = 0; ii < DKQ; ++ii)
-            if (ii < dkq) sp[(int64_t)(4 * ii + sub) * dv + col] = S[ii];
+            if (ii < dkq) sp[(int64_t)(SUBS * ii + sub) * dv + col] = S[ii];
     }
 }
 
@@ -160,13 +190,14 @@ __global__ __launch_bounds__(256) void delta_post_kernel(const float* __restrict
 
 }  // namespace
 
-extern "C" int32_t nvh_delta_prep(const void* k, int64_t k_stride, const void* a_raw, int64_t a_stride, const void* lowrank, int64_t lowrank_stride,
+extern "C" int32_t nvh_delta_prep(const void* r, int64_t r_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                                  const void* a_raw, int64_t a_stride, const void* lowrank, int64_t lowrank_stride,
                                   const void* w2, const void* w0, const void* a_bias, float* out, int64_t num_tokens, int64_t heads, int64_t dk,
                                   int64_t rank, float decay_scale, int32_t act_f32, nvh_stream_t stream) {
-    NVH_REQUIRE(k && a_raw && lowrank && w2 && w0 && a_bias && out, NVH_EINVAL, "nvh_delta_prep: null pointer");
+    NVH_REQUIRE(r && k && v && a_raw && lowrank && w2 && w0 && a_bias && out, NVH_EINVAL, "nvh_delta_prep: null pointer");
     NVH_REQUIRE(num_tokens >= 0 && heads > 0 && dk > 0 && rank > 0 && rank <= 8192, NVH_EINVAL, "nvh_delta_prep: bad sizes");
     if (num_tokens == 0) return NVH_OK;
-    DeltaPrepArgs p{k, k_stride, a_raw, a_stride, lowrank, lowrank_stride, w2, w0, a_bias, out, (int)heads, (int)dk, (int)rank, decay_scale};
+    DeltaPrepArgs p{r, k, v, r_stride, k_stride, v_stride, a_raw, a_stride, lowrank, lowrank_stride, w2, w0, a_bias, out, (int)heads, (int)dk, (int)rank, decay_scale};
     hipStream_t st = (hipStream_t)stream;
     const size_t lds = sizeof(float) * (size_t)rank;
     if (act_f32) delta_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
@@ -175,29 +206,43 @@ extern "C" int32_t nvh_delta_prep(const void* k, int64_t k_stride, const void* a
     return NVH_OK;
 }
 
-template <typename A>
+template <int DKQ, int SUBS>
+static void launch_delta_scan_as(const DeltaScanArgs& p, int64_t batch, hipStream_t st) {
+    constexpr int COLS = 256 / SUBS;
+    constexpr int CH = (5 * DKQ * SUBS + COLS + 255) / 256;
+    constexpr int TOK = (32 / CH) < 2 ? 2 : (32 / CH);
+    const dim3 grid((unsigned)batch, (unsigned)p.H, (unsigned)nvh_cdiv(p.dv, COLS));
+    const size_t lds = sizeof(float) * (size_t)TOK * (5 * p.dk + COLS);
+    delta_scan_kernel<DKQ, SUBS><<<grid, 256, lds, st>>>(p);
+}
+
 static int32_t launch_delta_scan(const DeltaScanArgs& p, int64_t batch, hipStream_t st) {
-    const dim3 grid((unsigned)batch, (unsigned)p.H, (unsigned)nvh_cdiv(p.dv, 64));
-    const size_t lds = sizeof(float) * (size_t)DTOK * (5 * p.dk + p.dv);
-    const int dkq = p.dk / 4;
-    if (dkq <= 8) delta_scan_kernel<A, 8><<<grid, 256, lds, st>>>(p);
-    else if (dkq <= 16) delta_scan_kernel<A, 16><<<grid, 256, lds, st>>>(p);
-    else if (dkq <= 32) delta_scan_kernel<A, 32><<<grid, 256, lds, st>>>(p);
-    else delta_scan_kernel<A, 64><<<grid, 256, lds, st>>>(p);
+    // (the choice depends on dk alone, so a sequence sees one summation order whatever the batch or the cut)
+    if (p.dk % 16 == 0) {
+        const int dkq = p.dk / 16;
+        if (dkq <= 2) launch_delta_scan_as<2, 16>(p, batch, st);
+        else if (dkq <= 4) launch_delta_scan_as<4, 16>(p, batch, st);
+        else if (dkq <= 8) launch_delta_scan_as<8, 16>(p, batch, st);
+        else launch_delta_scan_as<16, 16>(p, batch, st);
+    } else {
+        const int dkq = p.dk / 4;
+        if (dkq <= 8) launch_delta_scan_as<8, 4>(p, batch, st);
+        else if (dkq <= 16) launch_delta_scan_as<16, 4>(p, batch, st);
+        else if (dkq <= 32) launch_delta_scan_as<32, 4>(p, batch, st);
+        else launch_delta_scan_as<64, 4>(p, batch, st);
+    }
     NVH_CHECK_LAUNCH("nvh_delta_scan");
     return NVH_OK;
 }
 
-extern "C" int32_t nvh_delta_scan(const void* r, int64_t r_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
-                                  const float* wua, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
-                                  const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
-                                  int32_t act_f32, nvh_stream_t stream) {
-    NVH_REQUIRE(r && k && v && wua && state && slots && context_lens && out, NVH_EINVAL, "nvh_delta_scan: null pointer");
-    NVH_REQUIRE(batch >= 0 && heads > 0 && dk > 0 && dv > 0, NVH_EINVAL, "nvh_delta_scan: bad sizes");
+extern "C" int32_t nvh_delta_scan(const float* pack, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                                  const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, nvh_stream_t stream) {
+    NVH_REQUIRE(pack && state && slots && context_lens && out, NVH_EINVAL, "nvh_delta_scan: null pointer");
+    NVH_REQUIRE(batch >= 0 && heads > 0 && dk > 0, NVH_EINVAL, "nvh_delta_scan: bad sizes");
     NVH_REQUIRE(dk % 4 == 0 && dk <= 256, NVH_ENOSYS, "nvh_delta_scan: key size %ld must be a multiple of 4, at most 256", (long)dk);
     if (batch == 0) return NVH_OK;
-    DeltaScanArgs p{r, k, v, r_stride, k_stride, v_stride, wua, state, slots, cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dv};
-    return act_f32 ? launch_delta_scan<float>(p, batch, (hipStream_t)stream) : launch_delta_scan<bf16>(p, batch, (hipStream_t)stream);
+    DeltaScanArgs p{pack, state, slots, cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dk};
+    return launch_delta_scan(p, batch, (hipStream_t)stream);
 }
 
 extern "C" int32_t nvh_delta_post(const float* o, const void* norm_weight, const void* gate, int64_t gate_stride, void* y, int64_t y_stride,

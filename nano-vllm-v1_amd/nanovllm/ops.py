@@ -706,12 +706,13 @@ def delta_rule(r, k, v, a_raw, lowrank, w2, w0, a_bias, state, slots, cu_seqlens
     assert state.dtype == F32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dk, dk) and slots.dtype == torch.int32
     assert w2.is_contiguous() and w2.shape[0] == heads * dk and (cu_seqlens_q is None or cu_seqlens_q.dtype == torch.int32)
     rank = w2.shape[1]
-    wua = torch.empty(t, 3, heads * dk, dtype=F32, device=r.device)
-    _hip.call("nvh_delta_prep", k.data_ptr(), k.stride(0), a_raw.data_ptr(), a_raw.stride(0), lowrank.data_ptr(), lowrank.stride(0),
-              w2.data_ptr(), w0.data_ptr(), a_bias.data_ptr(), wua.data_ptr(), t, heads, dk, rank, float(decay_scale), f, _stream())
+    pack = torch.empty(t, heads, 6, dk, dtype=F32, device=r.device)
+    _hip.call("nvh_delta_prep", r.data_ptr(), r.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), a_raw.data_ptr(),
+              a_raw.stride(0), lowrank.data_ptr(), lowrank.stride(0), w2.data_ptr(), w0.data_ptr(), a_bias.data_ptr(), pack.data_ptr(),
+              t, heads, dk, rank, float(decay_scale), f, _stream())
     out = torch.empty(t, heads * dk, dtype=F32, device=r.device)
-    _hip.call("nvh_delta_scan", r.data_ptr(), r.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), wua.data_ptr(),
-              state.data_ptr(), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(), out.data_ptr(), batch, heads, dk, dk, f, _stream())
+    _hip.call("nvh_delta_scan", pack.data_ptr(), state.data_ptr(), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(),
+              out.data_ptr(), batch, heads, dk, _stream())
     return out
 
 
