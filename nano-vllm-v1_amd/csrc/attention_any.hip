@@ -276,6 +276,174 @@ __global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The same attention on the matrix cores, for bf16 caches with dim and vdim multiples of 16.  A workgroup is 64
+// consecutive queries of one (sequence, head): four waves of 16 queries, all walking the same 64-key tiles (K rows and
+// V transposed in LDS).  Per tile a wave forms S^T = K Q^T (lane: query lane%16, keys 4 (lane/16) + r of each 16-key
+// block), keeps max / sum / weights in fp32, and accumulates O^T = V^T P^T with the weights as the B operand - as two
+// bf16 terms, p = hi + lo, so a weight enters the product with 16 bits of mantissa and the sums stay fp32.  Tiles start
+// at key 0 and every query has its own running maximum, so the result of a query does not depend on the cut or the batch.
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+constexpr int MQ = 64, MK = 64;
+
+template <int NKS, int NVT>
+__global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+    int seq = -1, q0 = 0, qlen = 0, qbase = 0;
+    {
+        int tile = blockIdx.x;
+        for (int b = 0; b < a.batch; ++b) {
+            const int lo = a.cu_seqlens_q ? a.cu_seqlens_q[b] : b, hi = a.cu_seqlens_q ? a.cu_seqlens_q[b + 1] : b + 1;
+            const int tiles = (hi - lo + MQ - 1) / MQ;
+            if (tile < tiles) {
+                seq = b;
+                q0 = tile * MQ;
+                qlen = hi - lo;
+                qbase = lo;
+                break;
+            }
+            tile -= tiles;
+        }
+    }
+    if (seq < 0) return;
+    const int head = blockIdx.y, kvh = head / (a.H / a.G);
+    const int dim = a.dim, vdim = a.vdim, nks = dim >> 4, nvt = vdim >> 4;
+    const int klen = a.context_lens[seq], past = klen - qlen;
+    const int nq = min(MQ, qlen - q0);
+    const int kld = dim + 8, vld = MK + 8;                   // LDS row strides in elements (8-byte aligned rows)
+    bf16* ks = reinterpret_cast<bf16*>(smem_raw);            // [MK][dim + 8]
+    bf16* vt = ks + MK * kld;                                // [vdim][MK + 8]: V transposed
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fq = lane >> 4;
+    const int qrow = wave * 16 + fr;                         // this lane's query within the workgroup
+    const bool qok = qrow < nq;
+    const int qpos = past + q0 + qrow;
+    const int last_key = past + q0 + nq - 1;
+    const bf16* qg = (const bf16*)a.q + ((int64_t)(qbase + q0 + (qok ? qrow : 0)) * a.H + head) * dim;
+    s16x4 qf[NKS];
+#pragma unroll
+    for (int i = 0; i < NKS; ++i)
+        if (i < nks) qf[i] = *reinterpret_cast<const s16x4*>(qg + i * 16 + fq * 4);
+    f32x4 o[NVT];
+#pragma unroll
+    for (int i = 0; i < NVT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    const int32_t* table = a.block_tables + (int64_t)seq * a.table_stride;
+    const int wave_last = past + q0 + min(wave * 16 + 15, nq - 1);      // keys beyond it are masked for the whole wave
+    for (int k0 = 0; k0 <= last_key; k0 += MK) {
+        __syncthreads();
+        // stage K rows (8 elements per access) and V transposed
+        for (int i = tid; i < MK * (dim >> 3); i += 256) {
+            const int r = i / (dim >> 3), c = (i - r * (dim >> 3)) << 3, key = k0 + r;
+            bf16x8 v = {};
+            if (key <= last_key) {
+                const int64_t slot = (int64_t)table[key / a.page] * a.page + key % a.page;
+                v = *reinterpret_cast<const bf16x8*>((const bf16*)a.k_cache + (slot * a.G + kvh) * dim + c);
+            }
+            *reinterpret_cast<bf16x8*>(ks + r * kld + c) = v;
+        }
+        for (int i = tid; i < MK * (vdim >> 3); i += 256) {
+            const int r = i % MK, c = (i / MK) << 3, key = k0 + r;       // consecutive lanes: consecutive keys (conflict-free transposed writes)
+            bf16x8 v = {};
+            if (key <= last_key) {
+                const int64_t slot = (int64_t)table[key / a.page] * a.page + key % a.page;
+                v = *reinterpret_cast<const bf16x8*>((const bf16*)a.v_cache + (slot * a.G + kvh) * vdim + c);
+            }
+#pragma unroll
+            for (int e = 0; e < 8; ++e) vt[(c + e) * vld + r] = v[e];
+        }
+        __syncthreads();
+        if (k0 > wave_last) continue;                        // (wave-uniform; the barriers above are passed by all)
+        f32x4 sc[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+            f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int i = 0; i < NKS; ++i)
+                if (i < nks) {
+                    const s16x4 kf = *reinterpret_cast<const s16x4*>(ks + (kt * 16 + fr) * kld + i * 16 + fq * 4);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf, qf[i], acc, 0, 0, 0);
+                }
+            sc[kt] = acc;
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const bool ok = qok && k0 + kt * 16 + fq * 4 + r <= qpos;
+                sc[kt][r] = ok ? sc[kt][r] * a.scale : -INFINITY;
+                mx = fmaxf(mx, sc[kt][r]);
+            }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);
+        const float alpha = m_new == -INFINITY ? 1.f : expf(m_run - m_new);
+        float sum = 0.f;
+        s16x4 ph[4], pl[4];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float pv = sc[kt][r] == -INFINITY ? 0.f : expf(sc[kt][r] - m_new);
+                sum += pv;
+                const bf16 hi = (bf16)pv;
+                const bf16 lo = (bf16)(pv - (float)hi);
+                ph[kt][r] = __builtin_bit_cast(short, hi);
+                pl[kt][r] = __builtin_bit_cast(short, lo);
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+#pragma unroll
+        for (int i = 0; i < NVT; ++i)
+            if (i < nvt) {
+                f32x4 acc = o[i] * alpha;
+#pragma unroll
+                for (int kt = 0; kt < 4; ++kt) {
+                    const s16x4 vf = *reinterpret_cast<const s16x4*>(vt + (i * 16 + fr) * vld + kt * 16 + fq * 4);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, ph[kt], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pl[kt], acc, 0, 0, 0);
+                }
+                o[i] = acc;
+            }
+    }
+    // epilogue through LDS: [MQ][vdim] fp32, then turn back by the query's position, gate, store
+    __syncthreads();
+    float* os = reinterpret_cast<float*>(smem_raw);
+    const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
+#pragma unroll
+    for (int i = 0; i < NVT; ++i)
+        if (i < nvt)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) os[qrow * vdim + i * 16 + fq * 4 + r] = o[i][r] * inv_l;
+    __syncthreads();
+    for (int i = tid; i < nq * vdim; i += 256) {
+        const int r = i / vdim, col = i - r * vdim;
+        const int64_t tok = qbase + q0 + r;
+        float v = os[i];
+        if (a.v_freq) {
+            int partner, pair;
+            bool first;
+            pair_of(col, vdim, a.v_interleaved, partner, pair, first);
+            const float ov = os[r * vdim + partner];
+            const float ang = (float)(past + q0 + r) * a.v_freq[pair];
+            const float cs = cosf(ang), sn = sinf(ang);
+            v = first ? v * cs + ov * sn : v * cs - ov * sn;
+        }
+        const float g = a.gate ? a.gate[tok * a.H + head] : 1.0f;
+        ((bf16*)a.out)[(tok * a.H + head) * vdim + col] = (bf16)(v * g);
+    }
+}
+
+template <int NKS, int NVT>
+static void launch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st) {
+    const size_t tiles = sizeof(bf16) * ((size_t)MK * (a.dim + 8) + (size_t)a.vdim * (MK + 8));
+    const size_t outs = sizeof(float) * (size_t)MQ * a.vdim;
+    const dim3 grid((unsigned)(total_q / MQ + a.batch), (unsigned)a.H);
+    attn_paged_mfma_kernel<NKS, NVT><<<grid, 256, tiles > outs ? tiles : outs, st>>>(a);
+}
+
 }  // namespace
 
 extern "C" int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_stride, const void* q_norm_weight, const void* k_norm_weight,
@@ -319,8 +487,18 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     // at most ceil(len / AQ) tiles per sequence: total_q / AQ + batch bounds their number (surplus workgroups exit)
     const dim3 grid((unsigned)(total_q / AQ + batch), (unsigned)num_q_heads);
     hipStream_t st = (hipStream_t)stream;
-    if (act_f32) attn_paged_any_kernel<float><<<grid, 256, lds, st>>>(a);
-    else attn_paged_any_kernel<bf16><<<grid, 256, lds, st>>>(a);
+    // bf16 with 16-aligned head sizes: the matrix-core kernel (the choice depends on the sizes and the type only)
+    const bool mfma = !act_f32 && dim % 16 == 0 && vdim % 16 == 0 && dim <= 256 && vdim <= 256 && nvh_aligned16(q) && nvh_aligned16(k_cache) &&
+                      nvh_aligned16(v_cache) && !nvh_switch_on(SW_ATTN_ANY_NO_MFMA);
+    if (mfma) {
+        if (dim <= 64 && vdim <= 64) launch_attn_mfma<4, 4>(a, total_q, st);
+        else if (dim <= 128 && vdim <= 128) launch_attn_mfma<8, 8>(a, total_q, st);
+        else launch_attn_mfma<16, 16>(a, total_q, st);
+    } else if (act_f32) {
+        attn_paged_any_kernel<float><<<grid, 256, lds, st>>>(a);
+    } else {
+        attn_paged_any_kernel<bf16><<<grid, 256, lds, st>>>(a);
+    }
     NVH_CHECK_LAUNCH("nvh_attn_paged_any");
     return NVH_OK;
 }
