@@ -520,15 +520,16 @@ int32_t nvh_gemm_any_nt(const void* x, int64_t x_row_stride, const void* w, cons
  * dimensions of every q / k head are turned by position * qk_freq[pair] with cos and sin scaled by qk_mag (pairs are
  * (i, i + rot_dims/2), or (2i, 2i+1) when interleaved; the frequency table carries any scaling rule); the value is
  * turned by its position over all vdim dimensions with v_freq (NULL: stored as it is).  q -> q_out [T, H dim], k and v ->
- * cache rows slot_mapping[t] (slot < 0 or NULL caches: not stored), sigmoid(gate) -> gate_out fp32 [T, H]. */
+ * cache rows slot_mapping[t] (slot < 0 or NULL caches: not stored), sigmoid(gate) -> gate_out fp32 [T, H].
+ * Cache layouts: keys [pages, page, G, dim]; values transposed within a page, [pages, G, vdim, page]. */
 int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_stride, const void* q_norm_weight, const void* k_norm_weight,
                              float eps, const int64_t* positions, const float* qk_freq, float qk_mag, int64_t rot_dims,
                              int32_t qk_interleaved, const float* v_freq, int32_t v_interleaved, void* q_out, float* gate_out,
-                             void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t num_tokens,
+                             void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t page, int64_t num_tokens,
                              int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim, int32_t act_f32,
                              nvh_stream_t stream);
 /* Causal softmax attention of var-len queries (cu_seqlens_q NULL: one per sequence) over the paged caches
- * [pages, page, G, dim] / [pages, page, G, vdim]; context_lens counts the keys including this step's.  Scores, weights
+ * [pages, page, G, dim] / [pages, G, vdim, page]; context_lens counts the keys including this step's.  Scores, weights
  * and sums in fp32.  Epilogue: each head's output is turned back by the query's position (v_freq; NULL: none) and
  * multiplied by gate[t, h] (NULL: none).  out [T, H vdim] of type A. */
 int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const void* v_cache, const int32_t* cu_seqlens_q,

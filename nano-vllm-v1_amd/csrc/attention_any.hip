@@ -4,6 +4,9 @@
 //                         whole k projection (not per head), partial rotary on q and k (frequency table given by the
 //                         caller, so any scaling rule fits), rotation of the value by its own position over all of
 //                         vdim, sigmoid of the per-head gate; q goes to a packed buffer, k and v to their cache slots.
+//                         Keys are cached [pages, page, G, dim]; values TRANSPOSED within a page, [pages, G, vdim, page],
+//                         so the attention reads a value column over consecutive keys in one piece (its matrix
+//                         product wants V^T) and never transposes on the fly.
 //   nvh_attn_paged_any    softmax attention of var-len queries over the paged cache, scores / weights in fp32; the
 //                         epilogue turns each head's output back by the query's position and multiplies the gate.
 // Activations and caches are of type A (bf16 or fp32).  Key tiles always start at key 0 of a sequence and every query
@@ -53,9 +56,9 @@ struct PrepArgs {
     int v_interleaved;
     void* q_out;               // [T, H*dim]
     float* gate_out;           // [T, H], or null (no gate columns in proj)
-    void *k_cache, *v_cache;   // [slots, G*dim], [slots, G*vdim]
+    void *k_cache, *v_cache;   // [pages, page, G, dim], [pages, G, vdim, page] (values transposed within a page)
     const int32_t* slot_mapping;
-    int H, G, dim, vdim;
+    int H, G, dim, vdim, page;
 };
 
 template <typename A>
@@ -106,7 +109,7 @@ __global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
         }
     }
     if (slot >= 0 && a.v_cache) {
-        A* dst = (A*)a.v_cache + slot * nv;
+        A* dst = (A*)a.v_cache + (slot / a.page) * a.page * nv + slot % a.page;      // element i of the row goes to dst[i * page]
         for (int i = threadIdx.x; i < nv; i += 256) {
             float v = ldf(vr, i);
             if (a.v_freq) {
@@ -119,7 +122,7 @@ __global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
                 const float c = cosf(ang), s = sinf(ang);
                 v = first ? v * c - o * s : v * c + o * s;
             }
-            dst[i] = (A)v;
+            dst[(int64_t)i * a.page] = (A)v;
         }
     }
     if (a.gate_out)
@@ -205,8 +208,7 @@ __global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
             const int r = i / vdim, d = i - r * vdim, key = k0 + r;
             float v = 0.f;
             if (key <= last_key) {
-                const int64_t slot = (int64_t)table[key / a.page] * a.page + key % a.page;
-                v = ldf((const A*)a.v_cache, (slot * a.G + kvh) * vdim + d);
+                v = ldf((const A*)a.v_cache, (((int64_t)table[key / a.page] * a.G + kvh) * vdim + d) * a.page + key % a.page);
             }
             vs[r * vd + d] = v;
         }
@@ -328,31 +330,56 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     for (int i = 0; i < NVT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
     const int32_t* table = a.block_tables + (int64_t)seq * a.table_stride;
+    const bool wave_idle = wave * 16 >= nq;                  // no query of this wave is real (decode: three of four)
     const int wave_last = past + q0 + min(wave * 16 + 15, nq - 1);      // keys beyond it are masked for the whole wave
+    // A tile's global loads (16 bytes each; K rows as they lie, V rows = value columns over 64 consecutive keys of one page)
+    // are issued one tile ahead into registers; addresses are clamped, what lies beyond the last key is zeroed on the way
+    // into LDS.
+    constexpr int KCH = (NKS + 1) / 2, VCH = (NVT + 1) / 2;  // 16-byte pieces per lane: MK * dim / 8 / 256
+    bf16x8 kpre[KCH], vpre[VCH];
+    const int kcols = dim >> 3;
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < KCH; ++j) {
+            const int i = tid + 256 * j;
+            const int r = min(i / kcols, MK - 1), c = (i % kcols) << 3, key = min(k0 + r, last_key);
+            const int64_t slot = (int64_t)table[key / a.page] * a.page + key % a.page;
+            kpre[j] = *reinterpret_cast<const bf16x8*>((const bf16*)a.k_cache + (slot * a.G + kvh) * dim + c);
+        }
+        const int64_t vbase = ((int64_t)table[k0 / a.page] * a.G + kvh) * vdim;
+#pragma unroll
+        for (int j = 0; j < VCH; ++j) {
+            const int i = tid + 256 * j;
+            const int c = min(i >> 3, vdim - 1), piece = (i & 7) << 3;
+            vpre[j] = *reinterpret_cast<const bf16x8*>((const bf16*)a.v_cache + (vbase + c) * a.page + k0 % a.page + piece);
+        }
+    };
+    fetch(0);
     for (int k0 = 0; k0 <= last_key; k0 += MK) {
         __syncthreads();
-        // stage K rows (8 elements per access) and V transposed
-        for (int i = tid; i < MK * (dim >> 3); i += 256) {
-            const int r = i / (dim >> 3), c = (i - r * (dim >> 3)) << 3, key = k0 + r;
-            bf16x8 v = {};
-            if (key <= last_key) {
-                const int64_t slot = (int64_t)table[key / a.page] * a.page + key % a.page;
-                v = *reinterpret_cast<const bf16x8*>((const bf16*)a.k_cache + (slot * a.G + kvh) * dim + c);
-            }
-            *reinterpret_cast<bf16x8*>(ks + r * kld + c) = v;
-        }
-        for (int i = tid; i < MK * (vdim >> 3); i += 256) {
-            const int r = i % MK, c = (i / MK) << 3, key = k0 + r;       // consecutive lanes: consecutive keys (conflict-free transposed writes)
-            bf16x8 v = {};
-            if (key <= last_key) {
-                const int64_t slot = (int64_t)table[key / a.page] * a.page + key % a.page;
-                v = *reinterpret_cast<const bf16x8*>((const bf16*)a.v_cache + (slot * a.G + kvh) * vdim + c);
-            }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) vt[(c + e) * vld + r] = v[e];
+        for (int j = 0; j < KCH; ++j) {
+            const int i = tid + 256 * j;
+            if (i < MK * kcols) {
+                const int r = i / kcols, c = (i % kcols) << 3;
+                *reinterpret_cast<bf16x8*>(ks + r * kld + c) = k0 + r <= last_key ? kpre[j] : bf16x8{};
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VCH; ++j) {
+            const int i = tid + 256 * j;
+            if (i < vdim * 8) {
+                const int c = i >> 3, piece = (i & 7) << 3;
+                bf16x8 v = vpre[j];
+#pragma unroll
+                for (int e = 0; e < 8; ++e)
+                    if (k0 + piece + e > last_key) v[e] = (bf16)0.f;
+                *reinterpret_cast<bf16x8*>(vt + c * vld + piece) = v;
+            }
         }
         __syncthreads();
-        if (k0 > wave_last) continue;                        // (wave-uniform; the barriers above are passed by all)
+        if (k0 + MK <= last_key) fetch(k0 + MK);
+        if (wave_idle || k0 > wave_last) continue;           // (wave-uniform; the barriers above are passed by all)
         f32x4 sc[4];
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
@@ -449,11 +476,11 @@ static void launch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st)
 extern "C" int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_stride, const void* q_norm_weight, const void* k_norm_weight,
                                         float eps, const int64_t* positions, const float* qk_freq, float qk_mag, int64_t rot_dims,
                                         int32_t qk_interleaved, const float* v_freq, int32_t v_interleaved, void* q_out, float* gate_out,
-                                        void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t num_tokens,
+                                        void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t page, int64_t num_tokens,
                                         int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim, int32_t act_f32,
                                         nvh_stream_t stream) {
     NVH_REQUIRE(proj && q_norm_weight && k_norm_weight && positions && q_out, NVH_EINVAL, "nvh_attn_rotary_prep: null pointer");
-    NVH_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && dim > 0 && vdim > 0 && num_tokens >= 0, NVH_EINVAL, "nvh_attn_rotary_prep: bad sizes");
+    NVH_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && dim > 0 && vdim > 0 && num_tokens >= 0 && page > 0, NVH_EINVAL, "nvh_attn_rotary_prep: bad sizes");
     NVH_REQUIRE(rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0 && (rot_dims == 0 || qk_freq), NVH_EINVAL,
                 "nvh_attn_rotary_prep: rot_dims %ld does not fit dim %ld", (long)rot_dims, (long)dim);
     NVH_REQUIRE(!v_freq || vdim % 2 == 0, NVH_EINVAL, "nvh_attn_rotary_prep: rotated values need an even vdim");
@@ -461,7 +488,7 @@ extern "C" int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_strid
                 "nvh_attn_rotary_prep: projection row too short");
     if (num_tokens == 0) return NVH_OK;
     PrepArgs a{proj, proj_row_stride, q_norm_weight, k_norm_weight, eps, positions, qk_freq, qk_mag, (int)rot_dims, qk_interleaved,
-               v_freq, v_interleaved, q_out, gate_out, k_cache, v_cache, slot_mapping, (int)num_q_heads, (int)num_kv_heads, (int)dim, (int)vdim};
+               v_freq, v_interleaved, q_out, gate_out, k_cache, v_cache, slot_mapping, (int)num_q_heads, (int)num_kv_heads, (int)dim, (int)vdim, (int)page};
     hipStream_t st = (hipStream_t)stream;
     if (act_f32) attn_rotary_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(a);
     else attn_rotary_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(a);
@@ -488,7 +515,7 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     const dim3 grid((unsigned)(total_q / AQ + batch), (unsigned)num_q_heads);
     hipStream_t st = (hipStream_t)stream;
     // bf16 with 16-aligned head sizes: the matrix-core kernel (the choice depends on the sizes and the type only)
-    const bool mfma = !act_f32 && dim % 16 == 0 && vdim % 16 == 0 && dim <= 256 && vdim <= 256 && nvh_aligned16(q) && nvh_aligned16(k_cache) &&
+    const bool mfma = !act_f32 && dim % 16 == 0 && vdim % 16 == 0 && dim <= 256 && vdim <= 256 && page % MK == 0 && nvh_aligned16(q) && nvh_aligned16(k_cache) &&
                       nvh_aligned16(v_cache) && !nvh_switch_on(SW_ATTN_ANY_NO_MFMA);
     if (mfma) {
         if (dim <= 64 && vdim <= 64) launch_attn_mfma<4, 4>(a, total_q, st);

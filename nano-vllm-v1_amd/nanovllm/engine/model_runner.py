@@ -400,7 +400,7 @@ class ModelRunner:
         return sum(m.state_runs * slots * int(np.prod(m.state_shape())) * 4 for m in recurrent)
 
     def _bind_generic_caches(self, num_blocks: int, slots: int):
-        """Page caches [blocks, page, G, dim | vdim] per attention module and pass, fp32 state pools [slots, ...] per recurrent
+        """Page caches (keys [blocks, page, G, dim], values [blocks, G, vdim, page]) per attention module and pass, fp32 state pools [slots, ...] per recurrent
         module and pass (num_blocks 0: release them).  Nothing is cleared beyond allocation: keys are written before they are
         read, and a sequence's state is taken as zero in the step that brings its first tokens."""
         paged, recurrent = self._cache_modules()
@@ -408,7 +408,7 @@ class ModelRunner:
             for run in range(m.cache_runs):
                 if num_blocks:
                     m.k_caches[run] = torch.zeros(num_blocks, self.block_size, m.num_kv_heads, m.head_dim, dtype=self.dtype, device=self.device)
-                    m.v_caches[run] = torch.zeros(num_blocks, self.block_size, m.num_kv_heads, m.value_dim, dtype=self.dtype, device=self.device)
+                    m.v_caches[run] = torch.zeros(num_blocks, m.num_kv_heads, m.value_dim, self.block_size, dtype=self.dtype, device=self.device)
                 else:
                     m.k_caches[run] = m.v_caches[run] = None
         for m in recurrent:

@@ -72,7 +72,8 @@ class GatedValueRotaryAttention(nn.Module):
     Input is the fused projection output [T, H*dim + G*dim + G*vdim (+ H)] = q | k | v | gate; RMS norms over the WHOLE
     q and k projections run with the rotary in one launch (nvh_attn_rotary_prep), attention in a second
     (nvh_attn_paged_any).  A module that serves several passes of a looped stack owns one cache per pass:
-    `k_caches[run]`, `v_caches[run]`, views [pages, page, G, dim|vdim] bound by the runner (`cache_runs` of them)."""
+    `k_caches[run]` [pages, page, G, dim] and `v_caches[run]` [pages, G, vdim, page] (values lie transposed within a page),
+    bound by the runner (`cache_runs` of each)."""
 
     def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float, eps: float,
                  rot_dims: int, qk_freq: torch.Tensor, qk_mag: float, value_freq: torch.Tensor | None, gated: bool,

@@ -671,17 +671,19 @@ def attn_rotary_prep(proj, q_norm, k_norm, eps: float, positions, qk_freq, qk_ma
     gate = torch.empty(t, heads, dtype=F32, device=proj.device) if gated else None
     _hip.call("nvh_attn_rotary_prep", proj.data_ptr(), proj.stride(0), q_norm.data_ptr(), k_norm.data_ptr(), float(eps), positions.data_ptr(),
               _p(qk_freq), float(qk_mag), rot_dims, int(qk_interleaved), _p(v_freq), int(v_interleaved), q.data_ptr(), _p(gate),
-              k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(), t, heads, kv_heads, dim, vdim, f, _stream())
+              k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(), k_cache.shape[1], t, heads, kv_heads, dim, vdim, f, _stream())
     return q, gate
 
 
 def attn_paged_any(q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, scale: float, heads: int, kv_heads: int, dim: int,
                    vdim: int, gate=None, v_freq=None, v_interleaved: bool = False) -> torch.Tensor:
-    """Causal attention of the packed queries q [T, H*dim] over paged caches [pages, page, G, dim|vdim]; out [T, H*vdim]."""
+    """Causal attention of the packed queries q [T, H*dim] over paged caches, keys [pages, page, G, dim] and values
+    [pages, G, vdim, page] (transposed within a page, as attn_rotary_prep stores them); out [T, H*vdim]."""
     f = _act_flag(q, k_cache, v_cache)
     t = q.shape[0]
     batch = context_lens.numel()
     assert q.is_contiguous() and k_cache.is_contiguous() and v_cache.is_contiguous() and k_cache.dim() == 4
+    assert tuple(v_cache.shape) == (k_cache.shape[0], kv_heads, vdim, k_cache.shape[1])
     assert context_lens.dtype == torch.int32 and block_tables.dtype == torch.int32 and block_tables.stride(1) == 1
     assert cu_seqlens_q is None or (cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.numel() == batch + 1)
     assert cu_seqlens_q is not None or t == batch
