@@ -148,6 +148,8 @@ struct AttnArgs {
     const float* v_freq;       // [vdim/2] or null: no turning back
     int v_interleaved;
     void* out;                 // [T, H*vdim]
+    int fast_exp, no_lo;       // measurement switches (EXP_A, EXP_B)
+    int pages_offset;          // byte offset in LDS of the sequence's page ids (matrix-core kernel)
 };
 
 template <typename A>
@@ -288,7 +290,12 @@ __global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
 typedef short s16x4 __attribute__((ext_vector_type(4)));
 constexpr int MQ = 64, MK = 64;
 
-template <int NKS, int NVT>
+// EXACT: dim == 16 NKS and vdim == 16 NVT, so no loop below carries a run-time bound (a guarded loop body is a branch, and the
+// scheduler then cannot issue the LDS reads of several matrix instructions ahead of them).
+// GROUPED (steps in which every sequence brings one query): a workgroup is one (sequence, KV head) and the 16 query rows
+// of wave 0 are the query heads that share this KV head, so its keys and values are read once for all of them.  A row
+// goes through the same operations in the same order as in the other form: the bits are the same.
+template <int NKS, int NVT, bool EXACT, bool GROUPED>
 __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     int seq = -1, q0 = 0, qlen = 0, qbase = 0;
@@ -308,45 +315,63 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
         }
     }
     if (seq < 0) return;
-    const int head = blockIdx.y, kvh = head / (a.H / a.G);
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fq = lane >> 4;
+    const int group = a.H / a.G;
+    const int kvh = GROUPED ? blockIdx.y : blockIdx.y / group;
+    const int head = GROUPED ? kvh * group + min(fr, group - 1) : blockIdx.y;       // (GROUPED: this lane's row is a head)
     const int dim = a.dim, vdim = a.vdim, nks = dim >> 4, nvt = vdim >> 4;
     const int klen = a.context_lens[seq], past = klen - qlen;
-    const int nq = min(MQ, qlen - q0);
+    const int nq = GROUPED ? 1 : min(MQ, qlen - q0);
+    const int nrows = GROUPED ? group : nq;                  // real rows of the workgroup's 64
     const int kld = dim + 8, vld = MK + 8;                   // LDS row strides in elements (8-byte aligned rows)
     bf16* ks = reinterpret_cast<bf16*>(smem_raw);            // [MK][dim + 8]
     bf16* vt = ks + MK * kld;                                // [vdim][MK + 8]: V transposed
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fq = lane >> 4;
-    const int qrow = wave * 16 + fr;                         // this lane's query within the workgroup
-    const bool qok = qrow < nq;
-    const int qpos = past + q0 + qrow;
+    const int qrow = wave * 16 + fr;                         // this lane's row within the workgroup
+    const bool qok = qrow < nrows;
+    const int qpos = GROUPED ? past : past + q0 + qrow;
     const int last_key = past + q0 + nq - 1;
-    const bf16* qg = (const bf16*)a.q + ((int64_t)(qbase + q0 + (qok ? qrow : 0)) * a.H + head) * dim;
+    if (last_key < 0) {                                      // a padded row of a captured step (no keys): zeros, and no address is formed
+        for (int i = tid; i < nrows * vdim; i += 256) {
+            const int r = i / vdim;
+            const int64_t tok = GROUPED ? qbase : qbase + q0 + r;
+            const int hd = GROUPED ? kvh * group + r : (int)blockIdx.y;
+            ((bf16*)a.out)[(tok * a.H + hd) * vdim + (i - r * vdim)] = (bf16)0.f;
+        }
+        return;
+    }
+    const bf16* qg = (const bf16*)a.q + ((int64_t)(qbase + q0 + (qok && !GROUPED ? qrow : 0)) * a.H + head) * dim;
     s16x4 qf[NKS];
 #pragma unroll
     for (int i = 0; i < NKS; ++i)
-        if (i < nks) qf[i] = *reinterpret_cast<const s16x4*>(qg + i * 16 + fq * 4);
+        if (EXACT || i < nks) qf[i] = *reinterpret_cast<const s16x4*>(qg + i * 16 + fq * 4);
     f32x4 o[NVT];
 #pragma unroll
     for (int i = 0; i < NVT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
     const int32_t* table = a.block_tables + (int64_t)seq * a.table_stride;
-    const bool wave_idle = wave * 16 >= nq;                  // no query of this wave is real (decode: three of four)
-    const int wave_last = past + q0 + min(wave * 16 + 15, nq - 1);      // keys beyond it are masked for the whole wave
+    const bool wave_idle = wave * 16 >= nrows;               // no row of this wave is real
+    const int wave_last = GROUPED ? past : past + q0 + min(wave * 16 + 15, nq - 1);  // keys beyond it are masked for the whole wave
     // A tile's global loads (16 bytes each; K rows as they lie, V rows = value columns over 64 consecutive keys of one page)
     // are issued one tile ahead into registers; addresses are clamped, what lies beyond the last key is zeroed on the way
     // into LDS.
     constexpr int KCH = (NKS + 1) / 2, VCH = (NVT + 1) / 2;  // 16-byte pieces per lane: MK * dim / 8 / 256
     bf16x8 kpre[KCH], vpre[VCH];
     const int kcols = dim >> 3;
+    // The sequence's page ids go to LDS once: a tile's addresses then hang on no other load (a block-table read in front
+    // of every tile's loads doubled the latency a one-tile lead has to cover).  A tile lies within one page (page % MK == 0).
+    int* pages_s = reinterpret_cast<int*>(smem_raw + a.pages_offset);
+    for (int i = tid; i <= last_key / a.page; i += 256) pages_s[i] = table[i];
+    __syncthreads();
     auto fetch = [&](int k0) {
+        const int64_t pg = pages_s[k0 / a.page];
+        const int in_page = k0 % a.page, rows = last_key - k0;       // (uniform)
 #pragma unroll
         for (int j = 0; j < KCH; ++j) {
             const int i = tid + 256 * j;
-            const int r = min(i / kcols, MK - 1), c = (i % kcols) << 3, key = min(k0 + r, last_key);
-            const int64_t slot = (int64_t)table[key / a.page] * a.page + key % a.page;
-            kpre[j] = *reinterpret_cast<const bf16x8*>((const bf16*)a.k_cache + (slot * a.G + kvh) * dim + c);
+            const int r = min(min(i / kcols, MK - 1), rows), c = (i % kcols) << 3;
+            kpre[j] = *reinterpret_cast<const bf16x8*>((const bf16*)a.k_cache + (((pg * a.page + in_page + r) * a.G + kvh) * dim + c));
         }
-        const int64_t vbase = ((int64_t)table[k0 / a.page] * a.G + kvh) * vdim;
+        const int64_t vbase = (pg * a.G + kvh) * vdim;
 #pragma unroll
         for (int j = 0; j < VCH; ++j) {
             const int i = tid + 256 * j;
@@ -386,7 +411,7 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < NKS; ++i)
-                if (i < nks) {
+                if (EXACT || i < nks) {
                     const s16x4 kf = *reinterpret_cast<const s16x4*>(ks + (kt * 16 + fr) * kld + i * 16 + fq * 4);
                     acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf, qf[i], acc, 0, 0, 0);
                 }
@@ -411,7 +436,7 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
         for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float pv = sc[kt][r] == -INFINITY ? 0.f : expf(sc[kt][r] - m_new);
+                const float pv = sc[kt][r] == -INFINITY ? 0.f : (a.fast_exp ? __expf(sc[kt][r] - m_new) : expf(sc[kt][r] - m_new));
                 sum += pv;
                 const bf16 hi = (bf16)pv;
                 const bf16 lo = (bf16)(pv - (float)hi);
@@ -424,13 +449,13 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
         m_run = m_new;
 #pragma unroll
         for (int i = 0; i < NVT; ++i)
-            if (i < nvt) {
+            if (EXACT || i < nvt) {
                 f32x4 acc = o[i] * alpha;
 #pragma unroll
                 for (int kt = 0; kt < 4; ++kt) {
                     const s16x4 vf = *reinterpret_cast<const s16x4*>(vt + (i * 16 + fr) * vld + kt * 16 + fq * 4);
                     acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, ph[kt], acc, 0, 0, 0);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pl[kt], acc, 0, 0, 0);
+                    if (!a.no_lo) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pl[kt], acc, 0, 0, 0);
                 }
                 o[i] = acc;
             }
@@ -441,20 +466,21 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
 #pragma unroll
     for (int i = 0; i < NVT; ++i)
-        if (i < nvt)
+        if (EXACT || i < nvt)
 #pragma unroll
             for (int r = 0; r < 4; ++r) os[qrow * vdim + i * 16 + fq * 4 + r] = o[i][r] * inv_l;
     __syncthreads();
-    for (int i = tid; i < nq * vdim; i += 256) {
+    for (int i = tid; i < nrows * vdim; i += 256) {
         const int r = i / vdim, col = i - r * vdim;
-        const int64_t tok = qbase + q0 + r;
+        const int64_t tok = GROUPED ? qbase : qbase + q0 + r;
+        const int head = GROUPED ? kvh * group + r : (int)blockIdx.y;
         float v = os[i];
         if (a.v_freq) {
             int partner, pair;
             bool first;
             pair_of(col, vdim, a.v_interleaved, partner, pair, first);
             const float ov = os[r * vdim + partner];
-            const float ang = (float)(past + q0 + r) * a.v_freq[pair];
+            const float ang = (float)(GROUPED ? past : past + q0 + r) * a.v_freq[pair];
             const float cs = cosf(ang), sn = sinf(ang);
             v = first ? v * cs + ov * sn : v * cs - ov * sn;
         }
@@ -463,12 +489,36 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     }
 }
 
-template <int NKS, int NVT>
+template <int NKS, int NVT, bool EXACT>
 static void launch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st) {
     const size_t tiles = sizeof(bf16) * ((size_t)MK * (a.dim + 8) + (size_t)a.vdim * (MK + 8));
     const size_t outs = sizeof(float) * (size_t)MQ * a.vdim;
-    const dim3 grid((unsigned)(total_q / MQ + a.batch), (unsigned)a.H);
-    attn_paged_mfma_kernel<NKS, NVT><<<grid, 256, tiles > outs ? tiles : outs, st>>>(a);
+    AttnArgs b = a;
+    b.pages_offset = (int)(((tiles > outs ? tiles : outs) + 15) & ~(size_t)15);
+    const size_t lds = b.pages_offset + sizeof(int) * (size_t)a.table_stride;
+    const int group = a.H / a.G;
+    if (total_q == a.batch && group > 1 && group <= 16) {    // one query per sequence: the heads of a KV group share a workgroup
+        attn_paged_mfma_kernel<NKS, NVT, EXACT, true><<<dim3((unsigned)a.batch, (unsigned)a.G), 256, lds, st>>>(b);
+    } else {
+        const dim3 grid((unsigned)(total_q / MQ + a.batch), (unsigned)a.H);
+        attn_paged_mfma_kernel<NKS, NVT, EXACT, false><<<grid, 256, lds, st>>>(b);
+    }
+}
+
+// Exact instantiations for the head sizes in use (dim/16, vdim/16); any other 16-aligned pair takes a bounded one.
+#define NVH_ATTN_EXACT(X) X(1, 1) X(2, 2) X(3, 3) X(4, 4) X(5, 5) X(6, 6) X(8, 8) X(12, 12) X(16, 16) X(2, 4) X(4, 2) X(4, 8) X(8, 4) X(8, 16) X(16, 8) X(12, 8)
+static void dispatch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st) {
+    const int nks = a.dim / 16, nvt = a.vdim / 16;
+#define NVH_ATTN_CASE(K, V)                              \
+    if (nks == K && nvt == V) {                          \
+        launch_attn_mfma<K, V, true>(a, total_q, st);    \
+        return;                                          \
+    }
+    NVH_ATTN_EXACT(NVH_ATTN_CASE)
+#undef NVH_ATTN_CASE
+    if (nks <= 4 && nvt <= 4) launch_attn_mfma<4, 4, false>(a, total_q, st);
+    else if (nks <= 8 && nvt <= 8) launch_attn_mfma<8, 8, false>(a, total_q, st);
+    else launch_attn_mfma<16, 16, false>(a, total_q, st);
 }
 
 }  // namespace
@@ -510,7 +560,7 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     NVH_REQUIRE(lds <= 64 * 1024, NVH_ENOSYS, "nvh_attn_paged_any: dim %ld + vdim %ld need %zu bytes of LDS", (long)dim, (long)vdim, lds);
     if (batch == 0 || total_q == 0) return NVH_OK;
     AttnArgs a{q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, table_stride, (int)batch, (int)page, (int)num_q_heads,
-               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out};
+               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, (int)nvh_switch_on(SW_EXP_A), (int)nvh_switch_on(SW_EXP_B), 0};
     // at most ceil(len / AQ) tiles per sequence: total_q / AQ + batch bounds their number (surplus workgroups exit)
     const dim3 grid((unsigned)(total_q / AQ + batch), (unsigned)num_q_heads);
     hipStream_t st = (hipStream_t)stream;
@@ -518,9 +568,7 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     const bool mfma = !act_f32 && dim % 16 == 0 && vdim % 16 == 0 && dim <= 256 && vdim <= 256 && page % MK == 0 && nvh_aligned16(q) && nvh_aligned16(k_cache) &&
                       nvh_aligned16(v_cache) && !nvh_switch_on(SW_ATTN_ANY_NO_MFMA);
     if (mfma) {
-        if (dim <= 64 && vdim <= 64) launch_attn_mfma<4, 4>(a, total_q, st);
-        else if (dim <= 128 && vdim <= 128) launch_attn_mfma<8, 8>(a, total_q, st);
-        else launch_attn_mfma<16, 16>(a, total_q, st);
+        dispatch_attn_mfma(a, total_q, st);
     } else if (act_f32) {
         attn_paged_any_kernel<float><<<grid, 256, lds, st>>>(a);
     } else {

@@ -81,7 +81,8 @@ struct DeltaScanArgs {
 // Lanes per state column (SUBS: 16 when dk is a multiple of 16, else 4), rows i = SUBS * ii + sub held by lane `sub`; a
 // workgroup of 256 lanes owns 256 / SUBS columns of one (sequence, head).  Tokens are staged TOK at a time: the loads
 // of the next TOK tokens are in flight (in registers) while the current ones are walked from LDS.
-template <int DKQ, int SUBS>
+// EXACT: dk == DKQ * SUBS, so the loops over a lane's rows carry no run-time bound (see attention_any.hip).
+template <int DKQ, int SUBS, bool EXACT>
 __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
     constexpr int COLS = 256 / SUBS;
     constexpr int CH = (5 * DKQ * SUBS + COLS + 255) / 256;  // loads per lane and token
@@ -98,7 +99,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
     float* sp = p.state + (((int64_t)slot * p.H + head) * dk) * dv;
     float S[DKQ];
 #pragma unroll
-    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && ii < dkq) ? sp[(int64_t)(SUBS * ii + sub) * dv + col] : 0.f;
+    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && (EXACT || ii < dkq)) ? sp[(int64_t)(SUBS * ii + sub) * dv + col] : 0.f;
     const int rowf = 5 * dk + COLS;
     // Row of a token as this workgroup needs it: the five dk-vectors, then its COLS columns of v.  Every load is
     // unconditional (indices clamped into the row and into the sequence), so all of a round's loads are in flight together.
@@ -130,14 +131,30 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
             }
         __syncthreads();
         if (t0 + TOK < hi) fetch(t0 + TOK);
-        for (int tt = 0; tt < nt; ++tt) {
+        // A token's operands are read from LDS one token ahead, so the reads' latency is off the chain S -> dot -> S.
+        float cr[DKQ], ck[DKQ], cw[DKQ], cu[DKQ], ca[DKQ], cv;
+        auto read_token = [&](int tt, float (&xr)[DKQ], float (&xk)[DKQ], float (&xw)[DKQ], float (&xu)[DKQ], float (&xa)[DKQ], float& xv) {
             const float* row = sm + tt * rowf;
-            const float *rr = row, *kk = row + dk, *ww = row + 2 * dk, *uu = row + 3 * dk, *au = row + 4 * dk;
-            const float vj = row[5 * dk + lcol];
+#pragma unroll
+            for (int ii = 0; ii < DKQ; ++ii)
+                if (EXACT || ii < dkq) {
+                    const int i = SUBS * ii + sub;
+                    xr[ii] = row[i];
+                    xk[ii] = row[dk + i];
+                    xw[ii] = row[2 * dk + i];
+                    xu[ii] = row[3 * dk + i];
+                    xa[ii] = row[4 * dk + i];
+                }
+            xv = row[5 * dk + lcol];
+        };
+        read_token(0, cr, ck, cw, cu, ca, cv);
+        for (int tt = 0; tt < nt; ++tt) {
+            float nr[DKQ], nk[DKQ], nw[DKQ], nu[DKQ], na[DKQ], nv;
+            read_token(min(tt + 1, TOK - 1), nr, nk, nw, nu, na, nv);
             float dot = 0.f;
 #pragma unroll
             for (int ii = 0; ii < DKQ; ++ii)
-                if (ii < dkq) dot = __builtin_fmaf(uu[SUBS * ii + sub], S[ii], dot);
+                if (EXACT || ii < dkq) dot = __builtin_fmaf(cu[ii], S[ii], dot);
             if constexpr (SUBS == 16) {
                 dot = row16_sum(dot);
             } else {
@@ -147,11 +164,10 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
             float o = 0.f;
 #pragma unroll
             for (int ii = 0; ii < DKQ; ++ii)
-                if (ii < dkq) {
-                    const int i = SUBS * ii + sub;
-                    const float s = __builtin_fmaf(ww[i], S[ii], __builtin_fmaf(kk[i], vj, -(au[i] * dot)));
-                    S[ii] = s;
-                    o = __builtin_fmaf(s, rr[i], o);
+                if (EXACT || ii < dkq) {
+                    const float sn = __builtin_fmaf(cw[ii], S[ii], __builtin_fmaf(ck[ii], cv, -(ca[ii] * dot)));
+                    S[ii] = sn;
+                    o = __builtin_fmaf(sn, cr[ii], o);
                 }
             if constexpr (SUBS == 16) {
                 o = row16_sum(o);
@@ -160,12 +176,21 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
                 o += NVH_DPP(o, 0x4E);
             }
             if (live && sub == 0) p.out[(int64_t)(t0 + tt) * p.H * dv + head * dv + col] = o;
+#pragma unroll
+            for (int ii = 0; ii < DKQ; ++ii) {
+                cr[ii] = nr[ii];
+                ck[ii] = nk[ii];
+                cw[ii] = nw[ii];
+                cu[ii] = nu[ii];
+                ca[ii] = na[ii];
+            }
+            cv = nv;
         }
     }
     if (live) {
 #pragma unroll
         for (int ii = 0; ii < DKQ; ++ii)
-            if (ii < dkq) sp[(int64_t)(SUBS * ii + sub) * dv + col] = S[ii];
+            if (EXACT || ii < dkq) sp[(int64_t)(SUBS * ii + sub) * dv + col] = S[ii];
     }
 }
 
@@ -206,30 +231,37 @@ extern "C" int32_t nvh_delta_prep(const void* r, int64_t r_stride, const void* k
     return NVH_OK;
 }
 
-template <int DKQ, int SUBS>
+template <int DKQ, int SUBS, bool EXACT>
 static void launch_delta_scan_as(const DeltaScanArgs& p, int64_t batch, hipStream_t st) {
     constexpr int COLS = 256 / SUBS;
     constexpr int CH = (5 * DKQ * SUBS + COLS + 255) / 256;
     constexpr int TOK = (32 / CH) < 2 ? 2 : (32 / CH);
     const dim3 grid((unsigned)batch, (unsigned)p.H, (unsigned)nvh_cdiv(p.dv, COLS));
     const size_t lds = sizeof(float) * (size_t)TOK * (5 * p.dk + COLS);
-    delta_scan_kernel<DKQ, SUBS><<<grid, 256, lds, st>>>(p);
+    delta_scan_kernel<DKQ, SUBS, EXACT><<<grid, 256, lds, st>>>(p);
 }
 
 static int32_t launch_delta_scan(const DeltaScanArgs& p, int64_t batch, hipStream_t st) {
     // (the choice depends on dk alone, so a sequence sees one summation order whatever the batch or the cut)
     if (p.dk % 16 == 0) {
-        const int dkq = p.dk / 16;
-        if (dkq <= 2) launch_delta_scan_as<2, 16>(p, batch, st);
-        else if (dkq <= 4) launch_delta_scan_as<4, 16>(p, batch, st);
-        else if (dkq <= 8) launch_delta_scan_as<8, 16>(p, batch, st);
-        else launch_delta_scan_as<16, 16>(p, batch, st);
+        switch (p.dk / 16) {
+            case 1: launch_delta_scan_as<1, 16, true>(p, batch, st); break;
+            case 2: launch_delta_scan_as<2, 16, true>(p, batch, st); break;
+            case 3: launch_delta_scan_as<3, 16, true>(p, batch, st); break;
+            case 4: launch_delta_scan_as<4, 16, true>(p, batch, st); break;
+            case 6: launch_delta_scan_as<6, 16, true>(p, batch, st); break;
+            case 8: launch_delta_scan_as<8, 16, true>(p, batch, st); break;
+            case 16: launch_delta_scan_as<16, 16, true>(p, batch, st); break;
+            default:
+                if (p.dk / 16 <= 8) launch_delta_scan_as<8, 16, false>(p, batch, st);
+                else launch_delta_scan_as<16, 16, false>(p, batch, st);
+        }
     } else {
         const int dkq = p.dk / 4;
-        if (dkq <= 8) launch_delta_scan_as<8, 4>(p, batch, st);
-        else if (dkq <= 16) launch_delta_scan_as<16, 4>(p, batch, st);
-        else if (dkq <= 32) launch_delta_scan_as<32, 4>(p, batch, st);
-        else launch_delta_scan_as<64, 4>(p, batch, st);
+        if (dkq <= 8) launch_delta_scan_as<8, 4, false>(p, batch, st);
+        else if (dkq <= 16) launch_delta_scan_as<16, 4, false>(p, batch, st);
+        else if (dkq <= 32) launch_delta_scan_as<32, 4, false>(p, batch, st);
+        else launch_delta_scan_as<64, 4, false>(p, batch, st);
     }
     NVH_CHECK_LAUNCH("nvh_delta_scan");
     return NVH_OK;
