@@ -543,7 +543,7 @@ int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const void* v_cac
  * a = sigmoid(a_raw + a_bias), u = k / sqrt(sum_head k^2 + 1e-6) (value size = key size dk).
  * nvh_delta_scan: sequence b owns state slot slots[b] (< 0: a padded row) and this step's tokens cu_seqlens_q[b] ..
  * (NULL: row b); it starts from zero when context_lens[b] equals its token count, else from the slot, and leaves the
- * state there; out fp32 [T, H dk].  dk % 4 == 0, dk <= 256.
+ * state there; out fp32 [T, H dk].  dk <= 256.
  * nvh_delta_post: y (type A) = o / rms_head(o) * norm_weight * sigmoid(gate) (gate NULL: none). */
 int32_t nvh_delta_prep(const void* r, int64_t r_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
                        const void* a_raw, int64_t a_stride, const void* lowrank, int64_t lowrank_stride,

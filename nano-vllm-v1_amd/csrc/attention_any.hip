@@ -557,7 +557,12 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     NVH_REQUIRE(vdim <= 16 * AVC, NVH_ENOSYS, "nvh_attn_paged_any: vdim %ld above %d", (long)vdim, 16 * AVC);
     NVH_REQUIRE(!v_freq || vdim % 2 == 0, NVH_EINVAL, "nvh_attn_paged_any: rotated values need an even vdim");
     const size_t lds = sizeof(float) * (size_t)(AQ * dim + AK * (dim + 1) + AK * (vdim + 1) + AQ * AK);
-    NVH_REQUIRE(lds <= 64 * 1024, NVH_ENOSYS, "nvh_attn_paged_any: dim %ld + vdim %ld need %zu bytes of LDS", (long)dim, (long)vdim, lds);
+    NVH_REQUIRE(lds <= 160 * 1024, NVH_ENOSYS, "nvh_attn_paged_any: dim %ld + vdim %ld need %zu bytes of LDS", (long)dim, (long)vdim, lds);
+    if (lds > 64 * 1024) {                                   // beyond the default limit of dynamic LDS: raise it for both forms (gfx950: 160 KB per workgroup)
+        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_paged_any_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        const hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&attn_paged_any_kernel<bf16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        NVH_REQUIRE(e1 == hipSuccess && e2 == hipSuccess, NVH_ENOSYS, "nvh_attn_paged_any: %zu bytes of LDS refused", lds);
+    }
     if (batch == 0 || total_q == 0) return NVH_OK;
     AttnArgs a{q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, table_stride, (int)batch, (int)page, (int)num_q_heads,
                (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, (int)nvh_switch_on(SW_EXP_A), (int)nvh_switch_on(SW_EXP_B), 0};

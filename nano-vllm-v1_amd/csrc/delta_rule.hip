@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
     constexpr int TOK = (32 / CH) < 2 ? 2 : (32 / CH);
     extern __shared__ float sm[];                            // [TOK][5 dk + COLS]: r | k | w | u | au | v (this workgroup's columns)
     const int seq = blockIdx.x, head = blockIdx.y;
-    const int dk = p.dk, dv = p.dv, dkq = dk / SUBS;
+    const int dk = p.dk, dv = p.dv, dkq = (dk + SUBS - 1) / SUBS;      // rows i = SUBS * ii + sub >= dk (ragged dk) are held as zeros
     const int col0 = blockIdx.z * COLS, lcol = threadIdx.x / SUBS, col = col0 + lcol, sub = threadIdx.x % SUBS;
     const bool live = col < dv;
     const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
     float* sp = p.state + (((int64_t)slot * p.H + head) * dk) * dv;
     float S[DKQ];
 #pragma unroll
-    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && (EXACT || ii < dkq)) ? sp[(int64_t)(SUBS * ii + sub) * dv + col] : 0.f;
+    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && (EXACT || SUBS * ii + sub < dk)) ? sp[(int64_t)(SUBS * ii + sub) * dv + col] : 0.f;
     const int rowf = 5 * dk + COLS;
     // Row of a token as this workgroup needs it: the five dk-vectors, then its COLS columns of v.  Every load is
     // unconditional (indices clamped into the row and into the sequence), so all of a round's loads are in flight together.
@@ -139,11 +139,12 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
             for (int ii = 0; ii < DKQ; ++ii)
                 if (EXACT || ii < dkq) {
                     const int i = SUBS * ii + sub;
-                    xr[ii] = row[i];
-                    xk[ii] = row[dk + i];
-                    xw[ii] = row[2 * dk + i];
-                    xu[ii] = row[3 * dk + i];
-                    xa[ii] = row[4 * dk + i];
+                    const bool in = EXACT || i < dk;         // (a row beyond dk: all operands zero, its state stays zero)
+                    xr[ii] = in ? row[i] : 0.f;
+                    xk[ii] = in ? row[dk + i] : 0.f;
+                    xw[ii] = in ? row[2 * dk + i] : 0.f;
+                    xu[ii] = in ? row[3 * dk + i] : 0.f;
+                    xa[ii] = in ? row[4 * dk + i] : 0.f;
                 }
             xv = row[5 * dk + lcol];
         };
@@ -190,7 +191,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
     if (live) {
 #pragma unroll
         for (int ii = 0; ii < DKQ; ++ii)
-            if (EXACT || ii < dkq) sp[(int64_t)(SUBS * ii + sub) * dv + col] = S[ii];
+            if (EXACT || SUBS * ii + sub < dk) sp[(int64_t)(SUBS * ii + sub) * dv + col] = S[ii];
     }
 }
 
@@ -257,7 +258,7 @@ static int32_t launch_delta_scan(const DeltaScanArgs& p, int64_t batch, hipStrea
                 else launch_delta_scan_as<16, 16, false>(p, batch, st);
         }
     } else {
-        const int dkq = p.dk / 4;
+        const int dkq = (p.dk + 3) / 4;
         if (dkq <= 8) launch_delta_scan_as<8, 4, false>(p, batch, st);
         else if (dkq <= 16) launch_delta_scan_as<16, 4, false>(p, batch, st);
         else if (dkq <= 32) launch_delta_scan_as<32, 4, false>(p, batch, st);
@@ -271,7 +272,7 @@ extern "C" int32_t nvh_delta_scan(const float* pack, float* state, const int32_t
                                   const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, nvh_stream_t stream) {
     NVH_REQUIRE(pack && state && slots && context_lens && out, NVH_EINVAL, "nvh_delta_scan: null pointer");
     NVH_REQUIRE(batch >= 0 && heads > 0 && dk > 0, NVH_EINVAL, "nvh_delta_scan: bad sizes");
-    NVH_REQUIRE(dk % 4 == 0 && dk <= 256, NVH_ENOSYS, "nvh_delta_scan: key size %ld must be a multiple of 4, at most 256", (long)dk);
+    NVH_REQUIRE(dk <= 256, NVH_ENOSYS, "nvh_delta_scan: key size %ld above 256", (long)dk);
     if (batch == 0) return NVH_OK;
     DeltaScanArgs p{pack, state, slots, cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dk};
     return launch_delta_scan(p, batch, (hipStream_t)stream);

@@ -415,3 +415,22 @@ def test_temperature_zero_rows_take_the_maximum():
             for r in (0, 4, 5):
                 assert ids[r] == want[r]
             assert ids[2] == 17
+
+
+def test_sizes_no_kernel_tile_divides(tmp_path):
+    """A delta head size that is no multiple of 4, a width that is no multiple of 8, an odd decay rank, one KV head, and
+    attention heads of 256 (the largest the kernels take; fp32 serving needs more than the default 64 KB of LDS there)."""
+    cfg = {"architecture": "Lamutar", "vocab": 37, "width": 50, "norm": {"eps": 1e-6}, "logit_softcap": 3.0,
+           "loop": {"start": 0, "stop": 2, "times": 1},
+           "layers": [{"type": "general_delta", "mixer": {"heads": 3, "dim": 10}, "mlp": {"kind": "dense", "ff": 34}},
+                      {"type": "attention", "mixer": {"heads": 2, "kv_heads": 1, "dim": 256, "vdim": 256, "scale": 0.05,
+                                                      "rot": {"base": 777.0, "dims": 256, "scaling": {"factor": 8.0, "original": 32, "fast": 4.0, "slow": 0.5}}},
+                       "mlp": None}]}
+    case = Case(tmp_path, cfg, weights=random_weights(cfg, 6, ranks=(5,)))
+    toks = tokens_of(cfg, 80, 3)
+    for dtype in ("float32", "bfloat16"):
+        rp = case.replay(dtype)
+        try:
+            run_schedule(rp, case, {"a": toks, "b": toks[:7]}, [[("a", 33), ("b", 5)], [("a", 1), ("b", 2)], [("a", 46)]], dtype)
+        finally:
+            rp.close()
