@@ -148,8 +148,8 @@ struct AttnArgs {
     const float* v_freq;       // [vdim/2] or null: no turning back
     int v_interleaved;
     void* out;                 // [T, H*vdim]
-    int fast_exp, no_lo;       // measurement switches (EXP_A, EXP_B)
     int pages_offset;          // byte offset in LDS of the sequence's page ids (matrix-core kernel)
+    int ml_offset;             // ... and of the waves' (max, sum) pairs in the one-query form
 };
 
 template <typename A>
@@ -292,9 +292,10 @@ constexpr int MQ = 64, MK = 64;
 
 // EXACT: dim == 16 NKS and vdim == 16 NVT, so no loop below carries a run-time bound (a guarded loop body is a branch, and the
 // scheduler then cannot issue the LDS reads of several matrix instructions ahead of them).
-// GROUPED (steps in which every sequence brings one query): a workgroup is one (sequence, KV head) and the 16 query rows
-// of wave 0 are the query heads that share this KV head, so its keys and values are read once for all of them.  A row
-// goes through the same operations in the same order as in the other form: the bits are the same.
+// GROUPED (steps in which every sequence brings one query): a workgroup is one (sequence, KV head) and the 16 rows of a
+// wave are the query heads that share this KV head, so its keys and values are read once for all of them; the four
+// waves split every tile's keys and their partial results are merged at the end (the sums of a row are then formed in
+// another order than in the other form: equal within fp32 rounding, not bit for bit).
 template <int NKS, int NVT, bool EXACT, bool GROUPED>
 __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -326,8 +327,11 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     const int kld = dim + 8, vld = MK + 8;                   // LDS row strides in elements (8-byte aligned rows)
     bf16* ks = reinterpret_cast<bf16*>(smem_raw);            // [MK][dim + 8]
     bf16* vt = ks + MK * kld;                                // [vdim][MK + 8]: V transposed
-    const int qrow = wave * 16 + fr;                         // this lane's row within the workgroup
+    // GROUPED: every wave holds the same 16 rows (heads) and takes the 16 keys kt = wave of every 64-key tile, with its own
+    // running maximum, sum and output; the four partial results are merged at the end.
+    const int qrow = GROUPED ? fr : wave * 16 + fr;          // this lane's row within the workgroup
     const bool qok = qrow < nrows;
+    constexpr int NKT = GROUPED ? 1 : 4;                     // 16-key blocks of a tile per wave
     const int qpos = GROUPED ? past : past + q0 + qrow;
     const int last_key = past + q0 + nq - 1;
     if (last_key < 0) {                                      // a padded row of a captured step (no keys): zeros, and no address is formed
@@ -349,7 +353,7 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     for (int i = 0; i < NVT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
     const int32_t* table = a.block_tables + (int64_t)seq * a.table_stride;
-    const bool wave_idle = wave * 16 >= nrows;               // no row of this wave is real
+    const bool wave_idle = !GROUPED && wave * 16 >= nrows;   // no row of this wave is real
     const int wave_last = GROUPED ? past : past + q0 + min(wave * 16 + 15, nq - 1);  // keys beyond it are masked for the whole wave
     // A tile's global loads (16 bytes each; K rows as they lie, V rows = value columns over 64 consecutive keys of one page)
     // are issued one tile ahead into registers; addresses are clamped, what lies beyond the last key is zeroed on the way
@@ -396,18 +400,21 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
             if (i < vdim * 8) {
                 const int c = i >> 3, piece = (i & 7) << 3;
                 bf16x8 v = vpre[j];
+                if (k0 + MK - 1 > last_key) {                // (uniform: only the sequence's last tile)
 #pragma unroll
-                for (int e = 0; e < 8; ++e)
-                    if (k0 + piece + e > last_key) v[e] = (bf16)0.f;
+                    for (int e = 0; e < 8; ++e)
+                        if (k0 + piece + e > last_key) v[e] = (bf16)0.f;
+                }
                 *reinterpret_cast<bf16x8*>(vt + c * vld + piece) = v;
             }
         }
         __syncthreads();
         if (k0 + MK <= last_key) fetch(k0 + MK);
         if (wave_idle || k0 > wave_last) continue;           // (wave-uniform; the barriers above are passed by all)
-        f32x4 sc[4];
+        f32x4 sc[NKT];
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt) {
+        for (int t = 0; t < NKT; ++t) {
+            const int kt = GROUPED ? wave : t;
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < NKS; ++i)
@@ -415,33 +422,34 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
                     const s16x4 kf = *reinterpret_cast<const s16x4*>(ks + (kt * 16 + fr) * kld + i * 16 + fq * 4);
                     acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(kf, qf[i], acc, 0, 0, 0);
                 }
-            sc[kt] = acc;
+            sc[t] = acc;
         }
         float mx = -INFINITY;
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+        for (int t = 0; t < NKT; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const bool ok = qok && k0 + kt * 16 + fq * 4 + r <= qpos;
-                sc[kt][r] = ok ? sc[kt][r] * a.scale : -INFINITY;
-                mx = fmaxf(mx, sc[kt][r]);
+                const bool ok = qok && k0 + (GROUPED ? wave : t) * 16 + fq * 4 + r <= qpos;
+                sc[t][r] = ok ? sc[t][r] * a.scale : -INFINITY;
+                mx = fmaxf(mx, sc[t][r]);
             }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         const float m_new = fmaxf(m_run, mx);
-        const float alpha = m_new == -INFINITY ? 1.f : expf(m_run - m_new);
+        // e^x as the hardware's 2^(x log2 e): fp32 throughout, about 1 ulp
+        const float alpha = m_new == -INFINITY ? 1.f : __builtin_amdgcn_exp2f((m_run - m_new) * 1.4426950408889634f);
         float sum = 0.f;
-        s16x4 ph[4], pl[4];
+        s16x4 ph[NKT], pl[NKT];
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+        for (int t = 0; t < NKT; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const float pv = sc[kt][r] == -INFINITY ? 0.f : (a.fast_exp ? __expf(sc[kt][r] - m_new) : expf(sc[kt][r] - m_new));
+                const float pv = sc[t][r] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((sc[t][r] - m_new) * 1.4426950408889634f);
                 sum += pv;
                 const bf16 hi = (bf16)pv;
                 const bf16 lo = (bf16)(pv - (float)hi);
-                ph[kt][r] = __builtin_bit_cast(short, hi);
-                pl[kt][r] = __builtin_bit_cast(short, lo);
+                ph[t][r] = __builtin_bit_cast(short, hi);
+                pl[t][r] = __builtin_bit_cast(short, lo);
             }
         sum += __shfl_xor(sum, 16, 64);
         sum += __shfl_xor(sum, 32, 64);
@@ -452,10 +460,11 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
             if (EXACT || i < nvt) {
                 f32x4 acc = o[i] * alpha;
 #pragma unroll
-                for (int kt = 0; kt < 4; ++kt) {
+                for (int t = 0; t < NKT; ++t) {
+                    const int kt = GROUPED ? wave : t;
                     const s16x4 vf = *reinterpret_cast<const s16x4*>(vt + (i * 16 + fr) * vld + kt * 16 + fq * 4);
-                    acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, ph[kt], acc, 0, 0, 0);
-                    if (!a.no_lo) acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pl[kt], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, ph[t], acc, 0, 0, 0);
+                    acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pl[t], acc, 0, 0, 0);
                 }
                 o[i] = acc;
             }
@@ -463,12 +472,42 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     // epilogue through LDS: [MQ][vdim] fp32, then turn back by the query's position, gate, store
     __syncthreads();
     float* os = reinterpret_cast<float*>(smem_raw);
-    const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
+    if constexpr (GROUPED) {
+        // the four waves' partial results [wave][16 rows][vdim] and their (max, sum), merged into the first wave's rows
+        float* ml = reinterpret_cast<float*>(smem_raw + a.ml_offset);
 #pragma unroll
-    for (int i = 0; i < NVT; ++i)
-        if (EXACT || i < nvt)
+        for (int i = 0; i < NVT; ++i)
+            if (EXACT || i < nvt)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) os[qrow * vdim + i * 16 + fq * 4 + r] = o[i][r] * inv_l;
+                for (int r = 0; r < 4; ++r) os[(wave * 16 + fr) * vdim + i * 16 + fq * 4 + r] = o[i][r];
+        if (fq == 0) {
+            ml[(wave * 16 + fr) * 2] = m_run;
+            ml[(wave * 16 + fr) * 2 + 1] = l_run;
+        }
+        __syncthreads();
+        for (int i = tid; i < nrows * vdim; i += 256) {
+            const int r = i / vdim, col = i - r * vdim;
+            float big = -INFINITY;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) big = fmaxf(big, ml[(w * 16 + r) * 2]);
+            float num = 0.f, den = 0.f;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                const float mw = ml[(w * 16 + r) * 2];
+                const float f = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f((mw - big) * 1.4426950408889634f);
+                num += os[(w * 16 + r) * vdim + col] * f;
+                den += ml[(w * 16 + r) * 2 + 1] * f;
+            }
+            os[i] = den > 0.f ? num / den : 0.f;             // (element i of the first wave's rows: read above by this lane only)
+        }
+    } else {
+        const float inv_l = l_run > 0.f ? 1.0f / l_run : 0.f;
+#pragma unroll
+        for (int i = 0; i < NVT; ++i)
+            if (EXACT || i < nvt)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) os[qrow * vdim + i * 16 + fq * 4 + r] = o[i][r] * inv_l;
+    }
     __syncthreads();
     for (int i = tid; i < nrows * vdim; i += 256) {
         const int r = i / vdim, col = i - r * vdim;
@@ -495,7 +534,8 @@ static void launch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st)
     const size_t outs = sizeof(float) * (size_t)MQ * a.vdim;
     AttnArgs b = a;
     b.pages_offset = (int)(((tiles > outs ? tiles : outs) + 15) & ~(size_t)15);
-    const size_t lds = b.pages_offset + sizeof(int) * (size_t)a.table_stride;
+    b.ml_offset = (int)((b.pages_offset + sizeof(int) * (size_t)a.table_stride + 15) & ~(size_t)15);
+    const size_t lds = b.ml_offset + sizeof(float) * 4 * 16 * 2;
     const int group = a.H / a.G;
     if (total_q == a.batch && group > 1 && group <= 16) {    // one query per sequence: the heads of a KV group share a workgroup
         attn_paged_mfma_kernel<NKS, NVT, EXACT, true><<<dim3((unsigned)a.batch, (unsigned)a.G), 256, lds, st>>>(b);
@@ -565,7 +605,7 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     }
     if (batch == 0 || total_q == 0) return NVH_OK;
     AttnArgs a{q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, table_stride, (int)batch, (int)page, (int)num_q_heads,
-               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, (int)nvh_switch_on(SW_EXP_A), (int)nvh_switch_on(SW_EXP_B), 0};
+               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, 0, 0};
     // at most ceil(len / AQ) tiles per sequence: total_q / AQ + batch bounds their number (surplus workgroups exit)
     const dim3 grid((unsigned)(total_q / AQ + batch), (unsigned)num_q_heads);
     hipStream_t st = (hipStream_t)stream;
