@@ -98,8 +98,11 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
     const bool fresh = p.context_lens[seq] == hi - lo;
     float* sp = p.state + (((int64_t)slot * p.H + head) * dk) * dv;
     float S[DKQ];
+    // rows of a lane: DKQ consecutive ones when the sizes are exact (one 16-byte LDS read per operand and four rows), every
+    // SUBS-th one otherwise
+    auto row_of = [&](int ii) { return EXACT ? DKQ * sub + ii : SUBS * ii + sub; };
 #pragma unroll
-    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && (EXACT || SUBS * ii + sub < dk)) ? sp[(int64_t)(SUBS * ii + sub) * dv + col] : 0.f;
+    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && (EXACT || row_of(ii) < dk)) ? sp[(int64_t)row_of(ii) * dv + col] : 0.f;
     const int rowf = 5 * dk + COLS;
     // Row of a token as this workgroup needs it: the five dk-vectors, then its COLS columns of v.  Every load is
     // unconditional (indices clamped into the row and into the sequence), so all of a round's loads are in flight together.
@@ -135,10 +138,29 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
         float cr[DKQ], ck[DKQ], cw[DKQ], cu[DKQ], ca[DKQ], cv;
         auto read_token = [&](int tt, float (&xr)[DKQ], float (&xk)[DKQ], float (&xw)[DKQ], float (&xu)[DKQ], float (&xa)[DKQ], float& xv) {
             const float* row = sm + tt * rowf;
+            if constexpr (EXACT && DKQ % 4 == 0) {
+#pragma unroll
+                for (int c4 = 0; c4 < DKQ / 4; ++c4) {
+                    const int i = DKQ * sub + 4 * c4;
+                    const f32x4 vr = *reinterpret_cast<const f32x4*>(row + i), vk = *reinterpret_cast<const f32x4*>(row + dk + i),
+                                vw = *reinterpret_cast<const f32x4*>(row + 2 * dk + i), vu = *reinterpret_cast<const f32x4*>(row + 3 * dk + i),
+                                va = *reinterpret_cast<const f32x4*>(row + 4 * dk + i);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        xr[4 * c4 + e] = vr[e];
+                        xk[4 * c4 + e] = vk[e];
+                        xw[4 * c4 + e] = vw[e];
+                        xu[4 * c4 + e] = vu[e];
+                        xa[4 * c4 + e] = va[e];
+                    }
+                }
+                xv = row[5 * dk + lcol];
+                return;
+            }
 #pragma unroll
             for (int ii = 0; ii < DKQ; ++ii)
                 if (EXACT || ii < dkq) {
-                    const int i = SUBS * ii + sub;
+                    const int i = row_of(ii);
                     const bool in = EXACT || i < dk;         // (a row beyond dk: all operands zero, its state stays zero)
                     xr[ii] = in ? row[i] : 0.f;
                     xk[ii] = in ? row[dk + i] : 0.f;
@@ -148,14 +170,13 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
                 }
             xv = row[5 * dk + lcol];
         };
-        read_token(0, cr, ck, cw, cu, ca, cv);
-        for (int tt = 0; tt < nt; ++tt) {
-            float nr[DKQ], nk[DKQ], nw[DKQ], nu[DKQ], na[DKQ], nv;
-            read_token(min(tt + 1, TOK - 1), nr, nk, nw, nu, na, nv);
+        // one token: reads S, leaves the new S and the output (the operands were read one token ahead)
+        auto token = [&](int tt, const float (&xr)[DKQ], const float (&xk)[DKQ], const float (&xw)[DKQ], const float (&xu)[DKQ],
+                         const float (&xa)[DKQ], float xv) {
             float dot = 0.f;
 #pragma unroll
             for (int ii = 0; ii < DKQ; ++ii)
-                if (EXACT || ii < dkq) dot = __builtin_fmaf(cu[ii], S[ii], dot);
+                if (EXACT || ii < dkq) dot = __builtin_fmaf(xu[ii], S[ii], dot);
             if constexpr (SUBS == 16) {
                 dot = row16_sum(dot);
             } else {
@@ -166,9 +187,9 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
 #pragma unroll
             for (int ii = 0; ii < DKQ; ++ii)
                 if (EXACT || ii < dkq) {
-                    const float sn = __builtin_fmaf(cw[ii], S[ii], __builtin_fmaf(ck[ii], cv, -(ca[ii] * dot)));
+                    const float sn = __builtin_fmaf(xw[ii], S[ii], __builtin_fmaf(xk[ii], xv, -(xa[ii] * dot)));
                     S[ii] = sn;
-                    o = __builtin_fmaf(sn, cr[ii], o);
+                    o = __builtin_fmaf(sn, xr[ii], o);
                 }
             if constexpr (SUBS == 16) {
                 o = row16_sum(o);
@@ -177,21 +198,23 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
                 o += NVH_DPP(o, 0x4E);
             }
             if (live && sub == 0) p.out[(int64_t)(t0 + tt) * p.H * dv + head * dv + col] = o;
-#pragma unroll
-            for (int ii = 0; ii < DKQ; ++ii) {
-                cr[ii] = nr[ii];
-                ck[ii] = nk[ii];
-                cw[ii] = nw[ii];
-                cu[ii] = nu[ii];
-                ca[ii] = na[ii];
-            }
-            cv = nv;
+        };
+        // two register sets take turns (no copies): while one token is worked on, the next one's operands arrive
+        float nr[DKQ], nk[DKQ], nw[DKQ], nu[DKQ], na[DKQ], nv;
+        read_token(0, cr, ck, cw, cu, ca, cv);
+        int tt = 0;
+        for (; tt + 1 < nt; tt += 2) {
+            read_token(tt + 1, nr, nk, nw, nu, na, nv);
+            token(tt, cr, ck, cw, cu, ca, cv);
+            read_token(min(tt + 2, TOK - 1), cr, ck, cw, cu, ca, cv);
+            token(tt + 1, nr, nk, nw, nu, na, nv);
         }
+        if (tt < nt) token(tt, cr, ck, cw, cu, ca, cv);
     }
     if (live) {
 #pragma unroll
         for (int ii = 0; ii < DKQ; ++ii)
-            if (EXACT || SUBS * ii + sub < dk) sp[(int64_t)(SUBS * ii + sub) * dv + col] = S[ii];
+            if (EXACT || row_of(ii) < dk) sp[(int64_t)row_of(ii) * dv + col] = S[ii];
     }
 }
 
