@@ -29,6 +29,17 @@ __device__ __forceinline__ float block_sum_256(float v, float* scratch) {
     return scratch[0] + scratch[1] + scratch[2] + scratch[3];
 }
 
+// sin and cos of an fp32 angle through the hardware's sin(2 pi x) / cos(2 pi x): the turn count is reduced in float64 (an
+// angle of thousands of radians keeps its fp32 value exactly), the functions themselves are good to about 1e-6 absolute.
+// For the bf16 path; the library's sinf / cosf (used where everything is fp32) cost a few hundred instructions at such angles.
+__device__ __forceinline__ void sincos_turns(float ang, float& sn, float& cs) {
+    double rev = (double)ang * 0.15915494309189535;
+    rev -= floor(rev);
+    const float rf = (float)rev;
+    sn = __builtin_amdgcn_sinf(rf);
+    cs = __builtin_amdgcn_cosf(rf);
+}
+
 // Index of the rotation partner of element i among `n` rotated dimensions, and the pair number.
 __device__ __forceinline__ void pair_of(int i, int n, int interleaved, int& partner, int& pair, bool& first) {
     if (interleaved) {
@@ -296,18 +307,23 @@ constexpr int MQ = 64, MK = 64;
 // wave are the query heads that share this KV head, so its keys and values are read once for all of them; the four
 // waves split every tile's keys and their partial results are merged at the end (the sums of a row are then formed in
 // another order than in the other form: equal within fp32 rounding, not bit for bit).
-template <int NKS, int NVT, bool EXACT, bool GROUPED>
+// (The same split with 16 consecutive queries of one head as the rows was measured for prompts: no faster for one
+// 1024-token chunk, 1.7-1.9 x slower from two chunks on, because it stages K/V four times as often.  Not kept.)
+template <int NKS, int NVT, bool EXACT, int MODE>
 __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
+    constexpr bool GROUPED = MODE == 1;                      // rows are the heads of a KV group (one query per sequence)
+    constexpr bool SPLIT = MODE != 0;                        // the waves share 16 rows and split the keys
+    constexpr int ROWS_Q = MQ;                               // queries per workgroup
     extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
     int seq = -1, q0 = 0, qlen = 0, qbase = 0;
     {
         int tile = blockIdx.x;
         for (int b = 0; b < a.batch; ++b) {
             const int lo = a.cu_seqlens_q ? a.cu_seqlens_q[b] : b, hi = a.cu_seqlens_q ? a.cu_seqlens_q[b + 1] : b + 1;
-            const int tiles = (hi - lo + MQ - 1) / MQ;
+            const int tiles = (hi - lo + ROWS_Q - 1) / ROWS_Q;
             if (tile < tiles) {
                 seq = b;
-                q0 = tile * MQ;
+                q0 = tile * ROWS_Q;
                 qlen = hi - lo;
                 qbase = lo;
                 break;
@@ -322,16 +338,16 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     const int head = GROUPED ? kvh * group + min(fr, group - 1) : blockIdx.y;       // (GROUPED: this lane's row is a head)
     const int dim = a.dim, vdim = a.vdim, nks = dim >> 4, nvt = vdim >> 4;
     const int klen = a.context_lens[seq], past = klen - qlen;
-    const int nq = GROUPED ? 1 : min(MQ, qlen - q0);
+    const int nq = GROUPED ? 1 : min(ROWS_Q, qlen - q0);
     const int nrows = GROUPED ? group : nq;                  // real rows of the workgroup's 64
     const int kld = dim + 8, vld = MK + 8;                   // LDS row strides in elements (8-byte aligned rows)
     bf16* ks = reinterpret_cast<bf16*>(smem_raw);            // [MK][dim + 8]
     bf16* vt = ks + MK * kld;                                // [vdim][MK + 8]: V transposed
     // GROUPED: every wave holds the same 16 rows (heads) and takes the 16 keys kt = wave of every 64-key tile, with its own
     // running maximum, sum and output; the four partial results are merged at the end.
-    const int qrow = GROUPED ? fr : wave * 16 + fr;          // this lane's row within the workgroup
+    const int qrow = SPLIT ? fr : wave * 16 + fr;            // this lane's row within the workgroup
     const bool qok = qrow < nrows;
-    constexpr int NKT = GROUPED ? 1 : 4;                     // 16-key blocks of a tile per wave
+    constexpr int NKT = SPLIT ? 1 : 4;                       // 16-key blocks of a tile per wave
     const int qpos = GROUPED ? past : past + q0 + qrow;
     const int last_key = past + q0 + nq - 1;
     if (last_key < 0) {                                      // a padded row of a captured step (no keys): zeros, and no address is formed
@@ -353,20 +369,19 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
     for (int i = 0; i < NVT; ++i) o[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
     const int32_t* table = a.block_tables + (int64_t)seq * a.table_stride;
-    const bool wave_idle = !GROUPED && wave * 16 >= nrows;   // no row of this wave is real
-    const int wave_last = GROUPED ? past : past + q0 + min(wave * 16 + 15, nq - 1);  // keys beyond it are masked for the whole wave
+    const bool wave_idle = !SPLIT && wave * 16 >= nrows;     // no row of this wave is real
+    const int wave_last = SPLIT ? last_key : past + q0 + min(wave * 16 + 15, nq - 1);   // keys beyond it are masked for the whole wave
     // A tile's global loads (16 bytes each; K rows as they lie, V rows = value columns over 64 consecutive keys of one page)
-    // are issued one tile ahead into registers; addresses are clamped, what lies beyond the last key is zeroed on the way
+    // are issued two tiles ahead into registers; addresses are clamped, what lies beyond the last key is zeroed on the way
     // into LDS.
     constexpr int KCH = (NKS + 1) / 2, VCH = (NVT + 1) / 2;  // 16-byte pieces per lane: MK * dim / 8 / 256
-    bf16x8 kpre[KCH], vpre[VCH];
     const int kcols = dim >> 3;
-    // The sequence's page ids go to LDS once: a tile's addresses then hang on no other load (a block-table read in front
-    // of every tile's loads doubled the latency a one-tile lead has to cover).  A tile lies within one page (page % MK == 0).
+    // The sequence's page ids go to LDS once: a tile's addresses then hang on no other load.  A tile lies within one page
+    // (page % MK == 0).
     int* pages_s = reinterpret_cast<int*>(smem_raw + a.pages_offset);
     for (int i = tid; i <= last_key / a.page; i += 256) pages_s[i] = table[i];
     __syncthreads();
-    auto fetch = [&](int k0) {
+    auto fetch = [&](int k0, bf16x8 (&kpre)[KCH], bf16x8 (&vpre)[VCH]) {
         const int64_t pg = pages_s[k0 / a.page];
         const int in_page = k0 % a.page, rows = last_key - k0;       // (uniform)
 #pragma unroll
@@ -383,8 +398,11 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
             vpre[j] = *reinterpret_cast<const bf16x8*>((const bf16*)a.v_cache + (vbase + c) * a.page + k0 % a.page + piece);
         }
     };
-    fetch(0);
-    for (int k0 = 0; k0 <= last_key; k0 += MK) {
+    // Two register sets, two tiles ahead: the loads of tile t + 2 are issued when tile t has been handed to LDS.
+    bf16x8 kA[KCH], vA[VCH], kB[KCH], vB[VCH];
+    fetch(0, kA, vA);
+    if (MK <= last_key) fetch(MK, kB, vB);
+    auto tile = [&](int k0, bf16x8 (&kpre)[KCH], bf16x8 (&vpre)[VCH]) {
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < KCH; ++j) {
@@ -409,12 +427,12 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
             }
         }
         __syncthreads();
-        if (k0 + MK <= last_key) fetch(k0 + MK);
-        if (wave_idle || k0 > wave_last) continue;           // (wave-uniform; the barriers above are passed by all)
+        if (k0 + 2 * MK <= last_key) fetch(k0 + 2 * MK, kpre, vpre);
+        if (wave_idle || k0 > wave_last) return;             // (wave-uniform; the barriers above are passed by all)
         f32x4 sc[NKT];
 #pragma unroll
         for (int t = 0; t < NKT; ++t) {
-            const int kt = GROUPED ? wave : t;
+            const int kt = SPLIT ? wave : t;
             f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int i = 0; i < NKS; ++i)
@@ -429,7 +447,7 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
         for (int t = 0; t < NKT; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const bool ok = qok && k0 + (GROUPED ? wave : t) * 16 + fq * 4 + r <= qpos;
+                const bool ok = qok && k0 + (SPLIT ? wave : t) * 16 + fq * 4 + r <= qpos;
                 sc[t][r] = ok ? sc[t][r] * a.scale : -INFINITY;
                 mx = fmaxf(mx, sc[t][r]);
             }
@@ -461,18 +479,22 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
                 f32x4 acc = o[i] * alpha;
 #pragma unroll
                 for (int t = 0; t < NKT; ++t) {
-                    const int kt = GROUPED ? wave : t;
+                    const int kt = SPLIT ? wave : t;
                     const s16x4 vf = *reinterpret_cast<const s16x4*>(vt + (i * 16 + fr) * vld + kt * 16 + fq * 4);
                     acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, ph[t], acc, 0, 0, 0);
                     acc = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(vf, pl[t], acc, 0, 0, 0);
                 }
                 o[i] = acc;
             }
+    };
+    for (int k0 = 0; k0 <= last_key; k0 += 2 * MK) {
+        tile(k0, kA, vA);
+        if (k0 + MK <= last_key) tile(k0 + MK, kB, vB);
     }
     // epilogue through LDS: [MQ][vdim] fp32, then turn back by the query's position, gate, store
     __syncthreads();
     float* os = reinterpret_cast<float*>(smem_raw);
-    if constexpr (GROUPED) {
+    if constexpr (SPLIT) {
         // the four waves' partial results [wave][16 rows][vdim] and their (max, sum), merged into the first wave's rows
         float* ml = reinterpret_cast<float*>(smem_raw + a.ml_offset);
 #pragma unroll
@@ -509,22 +531,25 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
                 for (int r = 0; r < 4; ++r) os[qrow * vdim + i * 16 + fq * 4 + r] = o[i][r] * inv_l;
     }
     __syncthreads();
-    for (int i = tid; i < nrows * vdim; i += 256) {
-        const int r = i / vdim, col = i - r * vdim;
+    // one lane per rotation pair: both elements, one sine and cosine
+    const int half = vdim >> 1;
+    for (int i = tid; i < nrows * half; i += 256) {
+        const int r = i / half, pair = i - r * half;
+        const int c1 = a.v_interleaved ? 2 * pair : pair, c2 = a.v_interleaved ? 2 * pair + 1 : pair + half;
         const int64_t tok = GROUPED ? qbase : qbase + q0 + r;
-        const int head = GROUPED ? kvh * group + r : (int)blockIdx.y;
-        float v = os[i];
+        const int hd = GROUPED ? kvh * group + r : (int)blockIdx.y;
+        float u = os[r * vdim + c1], v = os[r * vdim + c2];
         if (a.v_freq) {
-            int partner, pair;
-            bool first;
-            pair_of(col, vdim, a.v_interleaved, partner, pair, first);
-            const float ov = os[r * vdim + partner];
-            const float ang = (float)(GROUPED ? past : past + q0 + r) * a.v_freq[pair];
-            const float cs = cosf(ang), sn = sinf(ang);
-            v = first ? v * cs + ov * sn : v * cs - ov * sn;
+            float sn, cs;
+            sincos_turns((float)(GROUPED ? past : past + q0 + r) * a.v_freq[pair], sn, cs);
+            const float u2 = u * cs + v * sn;                // the rotation by -position
+            v = v * cs - u * sn;
+            u = u2;
         }
-        const float g = a.gate ? a.gate[tok * a.H + head] : 1.0f;
-        ((bf16*)a.out)[(tok * a.H + head) * vdim + col] = (bf16)(v * g);
+        const float g = a.gate ? a.gate[tok * a.H + hd] : 1.0f;
+        bf16* dst = (bf16*)a.out + (tok * a.H + hd) * vdim;
+        dst[c1] = (bf16)(u * g);
+        dst[c2] = (bf16)(v * g);
     }
 }
 
@@ -537,11 +562,11 @@ static void launch_attn_mfma(const AttnArgs& a, int64_t total_q, hipStream_t st)
     b.ml_offset = (int)((b.pages_offset + sizeof(int) * (size_t)a.table_stride + 15) & ~(size_t)15);
     const size_t lds = b.ml_offset + sizeof(float) * 4 * 16 * 2;
     const int group = a.H / a.G;
-    if (total_q == a.batch && group > 1 && group <= 16) {    // one query per sequence: the heads of a KV group share a workgroup
-        attn_paged_mfma_kernel<NKS, NVT, EXACT, true><<<dim3((unsigned)a.batch, (unsigned)a.G), 256, lds, st>>>(b);
+    if (total_q == a.batch && group <= 16 && !nvh_switch_on(SW_EXP_A)) {      // one query per sequence: the heads of a KV group share a workgroup
+        attn_paged_mfma_kernel<NKS, NVT, EXACT, 1><<<dim3((unsigned)a.batch, (unsigned)a.G), 256, lds, st>>>(b);
     } else {
         const dim3 grid((unsigned)(total_q / MQ + a.batch), (unsigned)a.H);
-        attn_paged_mfma_kernel<NKS, NVT, EXACT, false><<<grid, 256, lds, st>>>(b);
+        attn_paged_mfma_kernel<NKS, NVT, EXACT, 0><<<grid, 256, lds, st>>>(b);
     }
 }
 
