@@ -40,6 +40,18 @@ __device__ __forceinline__ void sincos_turns(float ang, float& sn, float& cs) {
     cs = __builtin_amdgcn_cosf(rf);
 }
 
+// The rotation's sine and cosine for activations of type A: the library functions where everything is fp32, the hardware
+// path where the result is rounded to bf16 anyway.
+template <typename A>
+__device__ __forceinline__ void rot_sincos(float ang, float& sn, float& cs) {
+    if constexpr (sizeof(A) == 4) {
+        sn = sinf(ang);
+        cs = cosf(ang);
+    } else {
+        sincos_turns(ang, sn, cs);
+    }
+}
+
 // Index of the rotation partner of element i among `n` rotated dimensions, and the pair number.
 __device__ __forceinline__ void pair_of(int i, int n, int interleaved, int& partner, int& pair, bool& first) {
     if (interleaved) {
@@ -112,8 +124,9 @@ __global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
                 pair_of(d, a.rot_dims, a.qk_interleaved, partner, pair, first);
                 const int j = i - d + partner;
                 const float o = ldf(src, j) * inv * ldf(wn, j);
-                const float ang = pos * a.qk_freq[pair];
-                const float c = cosf(ang) * a.qk_mag, s = sinf(ang) * a.qk_mag;
+                float sn, cs;
+                rot_sincos<A>(pos * a.qk_freq[pair], sn, cs);
+                const float c = cs * a.qk_mag, s = sn * a.qk_mag;
                 v = first ? v * c - o * s : v * c + o * s;
             }
             dst[i] = (A)v;
@@ -129,8 +142,8 @@ __global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
                 bool first;
                 pair_of(d, a.vdim, a.v_interleaved, partner, pair, first);
                 const float o = ldf(vr, i - d + partner);
-                const float ang = pos * a.v_freq[pair];
-                const float c = cosf(ang), s = sinf(ang);
+                float s, c;
+                rot_sincos<A>(pos * a.v_freq[pair], s, c);
                 v = first ? v * c - o * s : v * c + o * s;
             }
             dst[(int64_t)i * a.page] = (A)v;
@@ -281,8 +294,8 @@ __global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
                     bool first;
                     pair_of(col, vdim, a.v_interleaved, partner, pair, first);
                     const float o = os[qi * vdim + partner];
-                    const float ang = pos * a.v_freq[pair];
-                    const float cs = cosf(ang), sn = sinf(ang);
+                    float sn, cs;
+                    rot_sincos<A>(pos * a.v_freq[pair], sn, cs);
                     v = first ? v * cs + o * sn : v * cs - o * sn;        // the rotation by -pos
                 }
                 ((A*)a.out)[(tok * a.H + head) * vdim + col] = (A)(v * g);

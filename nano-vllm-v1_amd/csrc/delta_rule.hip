@@ -41,7 +41,7 @@ __global__ __launch_bounds__(256) void delta_prep_kernel(DeltaPrepArgs p) {
     for (int r = threadIdx.x; r < p.rank; r += 256) tl[r] = tanhf(ldf((const A*)p.lowrank, t * p.l_stride + r));
     __syncthreads();
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, dk = p.dk;
-    for (int h = wave; h < p.H; h += 4) {
+    for (int h = blockIdx.y * 4 + wave; h < p.H; h += 4 * gridDim.y) {      // one head per wave; grid.y covers the heads four at a time
         float* out = p.out + (t * p.H + h) * 6 * dk;
         float ss = 0.f;
         for (int i = lane; i < dk; i += 64) {
@@ -249,8 +249,9 @@ extern "C" int32_t nvh_delta_prep(const void* r, int64_t r_stride, const void* k
     DeltaPrepArgs p{r, k, v, r_stride, k_stride, v_stride, a_raw, a_stride, lowrank, lowrank_stride, w2, w0, a_bias, out, (int)heads, (int)dk, (int)rank, decay_scale};
     hipStream_t st = (hipStream_t)stream;
     const size_t lds = sizeof(float) * (size_t)rank;
-    if (act_f32) delta_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
-    else delta_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, lds, st>>>(p);
+    const dim3 grid((unsigned)num_tokens, (unsigned)nvh_cdiv(heads, 4));
+    if (act_f32) delta_prep_kernel<float><<<grid, 256, lds, st>>>(p);
+    else delta_prep_kernel<bf16><<<grid, 256, lds, st>>>(p);
     NVH_CHECK_LAUNCH("nvh_delta_prep");
     return NVH_OK;
 }

@@ -18,31 +18,73 @@ struct DytNorm {            // tanh(alpha * x) * w + b; all three in the activat
     const void* b;
 };
 
+// tanh for the norm: the library's where everything is fp32; for bf16 results 1 - 2 / (e^2z + 1) on the hardware's 2^x and
+// reciprocal (about 1e-6 absolute; the result is rounded to 8 bits of mantissa).
 template <typename A>
-__device__ __forceinline__ float dyt_apply(const DytNorm& n, float alpha, float x, int c) {
-    return tanhf(alpha * x) * ldf((const A*)n.w, c) + ldf((const A*)n.b, c);
+__device__ __forceinline__ float dyt_tanh(float z) {
+    if constexpr (sizeof(A) == 4) {
+        return tanhf(z);
+    } else {
+        const float e = __builtin_amdgcn_exp2f(fminf(z, 20.f) * 2.8853900817779268f);        // e^(2z)
+        return 1.0f - 2.0f * __builtin_amdgcn_rcpf(e + 1.0f);
+    }
 }
 
 // x[row] = (accumulate ? x[row] : 0) + post(y[row]) + bias;  h[row] = next(x[row]).
 // y null: the stream is only normalised.  post / next with a null weight are skipped (next: no h written).
-template <typename A>
+// VEC: dim % 4 == 0 and every row 16-byte (A: 8-byte) aligned: four consecutive elements per lane, one access each.
+template <typename A, bool VEC>
 __global__ __launch_bounds__(256) void residual_dyt_kernel(const A* __restrict__ y, int64_t y_stride, DytNorm post, const A* __restrict__ bias,
                                                            float* __restrict__ x, int accumulate, DytNorm next, A* __restrict__ h,
                                                            int64_t h_stride, int dim) {
+    typedef A A4 __attribute__((ext_vector_type(4)));
     const int64_t row = blockIdx.x;
     const float pa = post.w ? ldf((const A*)post.alpha, 0) : 0.f;
     const float na = next.w ? ldf((const A*)next.alpha, 0) : 0.f;
     float* xr = x + row * dim;
-    for (int c = threadIdx.x; c < dim; c += 256) {
-        float s = accumulate ? xr[c] : 0.f;
-        if (y) {
-            float t = ldf(y, row * y_stride + c);
-            if (post.w) t = dyt_apply<A>(post, pa, t, c);
-            s += t;
+    constexpr int W = VEC ? 4 : 1;
+    for (int c = threadIdx.x * W; c < dim; c += 256 * W) {
+        float s[W], t[W], bv[W], pw[W], pb[W], nw[W], nb[W];
+        if constexpr (VEC) {
+            const f32x4 xv = accumulate ? *reinterpret_cast<const f32x4*>(xr + c) : f32x4{0.f, 0.f, 0.f, 0.f};
+            const A4 zero = {(A)0.f, (A)0.f, (A)0.f, (A)0.f};
+            const A4 yv = y ? *reinterpret_cast<const A4*>(y + row * y_stride + c) : zero;
+            const A4 b4 = bias ? *reinterpret_cast<const A4*>(bias + c) : zero;
+            const A4 pw4 = post.w ? *reinterpret_cast<const A4*>((const A*)post.w + c) : zero, pb4 = post.w ? *reinterpret_cast<const A4*>((const A*)post.b + c) : zero;
+            const A4 nw4 = next.w ? *reinterpret_cast<const A4*>((const A*)next.w + c) : zero, nb4 = next.w ? *reinterpret_cast<const A4*>((const A*)next.b + c) : zero;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                s[e] = xv[e];
+                t[e] = (float)yv[e];
+                bv[e] = (float)b4[e];
+                pw[e] = (float)pw4[e];
+                pb[e] = (float)pb4[e];
+                nw[e] = (float)nw4[e];
+                nb[e] = (float)nb4[e];
+            }
+        } else {
+            s[0] = accumulate ? xr[c] : 0.f;
+            t[0] = y ? ldf(y, row * y_stride + c) : 0.f;
+            bv[0] = bias ? ldf(bias, c) : 0.f;
+            pw[0] = post.w ? ldf((const A*)post.w, c) : 0.f;
+            pb[0] = post.w ? ldf((const A*)post.b, c) : 0.f;
+            nw[0] = next.w ? ldf((const A*)next.w, c) : 0.f;
+            nb[0] = next.w ? ldf((const A*)next.b, c) : 0.f;
         }
-        if (bias) s += ldf(bias, c);
-        if (y || bias) xr[c] = s;
-        if (next.w) h[row * h_stride + c] = (A)dyt_apply<A>(next, na, s, c);
+        float hv[W];
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            if (y) s[e] += post.w ? dyt_tanh<A>(pa * t[e]) * pw[e] + pb[e] : t[e];
+            s[e] += bv[e];
+            hv[e] = next.w ? dyt_tanh<A>(na * s[e]) * nw[e] + nb[e] : 0.f;
+        }
+        if constexpr (VEC) {
+            if (y || bias) *reinterpret_cast<f32x4*>(xr + c) = f32x4{s[0], s[1], s[2], s[3]};
+            if (next.w) *reinterpret_cast<A4*>(h + row * h_stride + c) = A4{(A)hv[0], (A)hv[1], (A)hv[2], (A)hv[3]};
+        } else {
+            if (y || bias) xr[c] = s[0];
+            if (next.w) h[row * h_stride + c] = (A)hv[0];
+        }
     }
 }
 
@@ -236,8 +278,18 @@ extern "C" int32_t nvh_residual_dyt(const void* y, int64_t y_stride, const void*
     if (rows == 0) return NVH_OK;
     hipStream_t st = (hipStream_t)stream;
     const DytNorm post{post_alpha, post_w, post_b}, next{next_alpha, next_w, next_b};
-    if (act_f32) residual_dyt_kernel<float><<<dim3((unsigned)rows), 256, 0, st>>>((const float*)y, y_stride, post, (const float*)bias, x, accumulate, next, (float*)h, h_stride, (int)dim);
-    else residual_dyt_kernel<bf16><<<dim3((unsigned)rows), 256, 0, st>>>((const bf16*)y, y_stride, post, (const bf16*)bias, x, accumulate, next, (bf16*)h, h_stride, (int)dim);
+    const int esz = act_f32 ? 4 : 2;
+    auto al = [&](const void* p, int bytes) { return p == nullptr || ((uintptr_t)p % bytes) == 0; };
+    const bool vec = dim % 4 == 0 && al(x, 16) && al(y, 4 * esz) && y_stride % 4 == 0 && al(h, 4 * esz) && h_stride % 4 == 0 && al(bias, 4 * esz) &&
+                     al(post_w, 4 * esz) && al(post_b, 4 * esz) && al(next_w, 4 * esz) && al(next_b, 4 * esz);
+    const dim3 grid((unsigned)rows);
+    if (act_f32) {
+        if (vec) residual_dyt_kernel<float, true><<<grid, 256, 0, st>>>((const float*)y, y_stride, post, (const float*)bias, x, accumulate, next, (float*)h, h_stride, (int)dim);
+        else residual_dyt_kernel<float, false><<<grid, 256, 0, st>>>((const float*)y, y_stride, post, (const float*)bias, x, accumulate, next, (float*)h, h_stride, (int)dim);
+    } else {
+        if (vec) residual_dyt_kernel<bf16, true><<<grid, 256, 0, st>>>((const bf16*)y, y_stride, post, (const bf16*)bias, x, accumulate, next, (bf16*)h, h_stride, (int)dim);
+        else residual_dyt_kernel<bf16, false><<<grid, 256, 0, st>>>((const bf16*)y, y_stride, post, (const bf16*)bias, x, accumulate, next, (bf16*)h, h_stride, (int)dim);
+    }
     NVH_CHECK_LAUNCH("nvh_residual_dyt");
     return NVH_OK;
 }
