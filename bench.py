@@ -465,7 +465,7 @@ HYBRID_SIZES = {
 
 
 def hybrid_compare(args):
-    """--hybrid-compare: prefill and decode throughput of the Lamutar design (attention and delta-rule layers 1:2, fp32 residual
+    """--hybrid-compare: prefill and decode throughput of the Lamutar design (delta-rule and attention layers in turn, fp32 residual
     stream, operator modules + captured decode graphs) beside Qwen3 (the closest model the engine serves: native executor)
     at equal width, heads, feed-forward size, depth and vocabulary; random weights, bf16.  One JSON line."""
     import tempfile
@@ -475,11 +475,11 @@ def hybrid_compare(args):
     def lamutar_cfg(z):
         attn = {"type": "attention", "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["head_dim"], "vdim": z["head_dim"],
                                                "scale": z["head_dim"] ** -0.5,
-                                               "rot": {"base": 1e6, "dims": z["head_dim"] // 2, "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}},
+                                               "rot": {"base": 1e6, "dims": z["head_dim"] // 2, "scaling": {"factor": 4.0, "original": 4096, "fast": 16.0, "slow": 2.0}}},
                 "mlp": {"kind": "dense", "ff": z["ff"]}}
         delta = {"type": "general_delta", "mixer": {"heads": z["width"] // 64, "dim": 64}, "mlp": {"kind": "dense", "ff": z["ff"]}}
         return {"architecture": "Lamutar", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "loop": None,
-                "layers": [attn if i % 3 == 0 else delta for i in range(z["layers"])]}
+                "layers": [attn if i % 2 == 1 else delta for i in range(z["layers"])]}
 
     def qwen3_cfg(z):
         return {"architectures": ["Qwen3ForCausalLM"], "hidden_size": z["width"], "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],

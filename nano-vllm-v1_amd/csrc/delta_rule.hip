@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
     for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && (EXACT || row_of(ii) < dk)) ? sp[(int64_t)row_of(ii) * dv + col] : 0.f;
     const int rowf = 5 * dk + COLS;
     // Row of a token as this workgroup needs it: the five dk-vectors, then its COLS columns of v.  Every load is
-    // unconditional (indices clamped into the row and into the sequence), so all of a round's loads are in flight together.
+    // unconditional (indices clamped into the row and into the sequence), so all of a stage's loads are in flight together.
     float pre[TOK][CH];
     const float* base = p.pack + (int64_t)head * 6 * dk;
     const int64_t tok_stride = (int64_t)p.H * 6 * dk;
@@ -124,7 +124,7 @@ __global__ __launch_bounds__(256) void delta_scan_kernel(DeltaScanArgs p) {
     fetch(lo);
     for (int t0 = lo; t0 < hi; t0 += TOK) {
         const int nt = min(TOK, hi - t0);
-        __syncthreads();                                     // the previous round's readers are done
+        __syncthreads();                                     // the previous stage's readers are done
 #pragma unroll
         for (int tt = 0; tt < TOK; ++tt)
 #pragma unroll

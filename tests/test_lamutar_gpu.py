@@ -30,7 +30,7 @@ CFG_LOOP = {"architecture": "Lamutar", "vocab": 131, "width": 96, "norm": {"eps"
             "loop": {"start": 1, "stop": 3, "times": 3}, "layers": [DELTA_A, ATTN_A, DELTA_B, ATTN_B]}
 CFG_FLAT = {"architecture": "Lamutar", "vocab": 200, "width": 128, "norm": {"eps": 1e-6}, "logit_softcap": None, "loop": None,
             "layers": [{"type": "attention", "mixer": {"heads": 2, "kv_heads": 1, "dim": 128, "vdim": 64, "scale": 0.09,
-                                                       "rot": {"base": 1e6, "dims": 64, "scaling": {"factor": 2.0, "original": 256, "fast": 32.0, "slow": 1.0}}},
+                                                       "rot": {"base": 1e6, "dims": 64, "scaling": {"factor": 3.0, "original": 256, "fast": 24.0, "slow": 2.0}}},
                         "mlp": {"kind": "dense", "ff": 256}},
                        {"type": "general_delta", "mixer": {"heads": 2, "dim": 64}, "mlp": {"kind": "dense", "ff": 256}}]}
 
