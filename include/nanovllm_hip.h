@@ -516,7 +516,7 @@ int32_t nvh_gemm_any_nt(const void* x, int64_t x_row_stride, const void* w, cons
 
 /* Attention with a norm over the whole projection, partial rotary, rotated values and a per-head output gate.
  * nvh_attn_rotary_prep reads the fused projection row [q (H dim) | k (G dim) | v (G vdim) | gate (H, when gate_out)] of
- * every token: RMS norm (eps, weights of the full projection size) over all of q and all of k; the first rot_dims
+ * every token: RMS norm (eps, weights of the full projection size; both NULL: no norm) over all of q and all of k; the first rot_dims
  * dimensions of every q / k head are turned by position * qk_freq[pair] with cos and sin scaled by qk_mag (pairs are
  * (i, i + rot_dims/2), or (2i, 2i+1) when interleaved; the frequency table carries any scaling rule); the value is
  * turned by its position over all vdim dimensions with v_freq (NULL: stored as it is).  q -> q_out [T, H dim], k and v ->
@@ -531,12 +531,15 @@ int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_stride, const vo
 /* Causal softmax attention of var-len queries (cu_seqlens_q NULL: one per sequence) over the paged caches
  * [pages, page, G, dim] / [pages, G, vdim, page]; context_lens counts the keys including this step's.  Scores, weights
  * and sums in fp32.  Epilogue: each head's output is turned back by the query's position (v_freq; NULL: none) and
- * multiplied by gate[t, h] (NULL: none).  out [T, H vdim] of type A. */
+ * multiplied by gate[t, h] (NULL: none).  out [T, H vdim] of type A.
+ * slopes (fp32 [H], NULL: none): a distance bias, score -= slopes[h] * (query position - key position).
+ * window > 0: query i sees key j <= i only when i - j < window or j < keep_first (the first tokens stay visible and
+ * their distance is counted from where they stand); key tiles no query of a workgroup can see are skipped.  window 0: plain causal attention. */
 int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const void* v_cache, const int32_t* cu_seqlens_q,
                            const int32_t* context_lens, const int32_t* block_tables, int64_t table_stride, int64_t batch,
                            int64_t total_q, int64_t page, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
-                           float scale, const float* gate, const float* v_freq, int32_t v_interleaved, void* out,
-                           int32_t act_f32, nvh_stream_t stream);
+                           float scale, const float* gate, const float* v_freq, int32_t v_interleaved, const float* slopes,
+                           int64_t window, int64_t keep_first, void* out, int32_t act_f32, nvh_stream_t stream);
 
 /* Generalized delta rule, state [slots, H, dk, dv] fp32:  S <- diag(w) S - (a u)(u^T S) + k v^T,  o = S^T r.
  * nvh_delta_prep: out fp32 [T, H, 6, dk] = r | k | w | u | a u | v per head, with w = exp(-decay_scale sigmoid(w0 + w2 tanh(lowrank))),
@@ -553,6 +556,81 @@ int32_t nvh_delta_scan(const float* pack, float* state, const int32_t* slots, co
                        const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, nvh_stream_t stream);
 int32_t nvh_delta_post(const float* o, const void* norm_weight, const void* gate, int64_t gate_stride, void* y, int64_t y_stride,
                        int64_t rows, int64_t heads, int64_t dv, float eps, int32_t act_f32, nvh_stream_t stream);
+
+/* x[T, dim] fp32 = table[ids] * scale + pos_table[positions] (pos_table NULL: no position term; ids / positions outside
+ * their tables contribute zeros). */
+int32_t nvh_embedding_pos_stream(const int64_t* ids, const int64_t* positions, const void* table, const void* pos_table, float scale,
+                                 float* x, int64_t num_tokens, int64_t dim, int64_t vocab, int64_t max_positions, int32_t act_f32,
+                                 nvh_stream_t stream);
+/* The close of a layer whose sublayers all read one norm of the stream, fused with the norm that opens the next layer.  Per row:
+ *   s = branch_scale * (unit(a) a_weight + unit(b) b_weight) + c + c32;   x <- x + s;   h <- norm(x)
+ * unit(v) = v / sqrt(mean(v^2) + branch_eps) for a branch with a weight, v itself for one without; NULL terms are skipped
+ * (a, b, c of type A, c32 fp32).  norm_kind 1: layer norm ((x - mean) / sqrt(var + eps) w + b, bias NULL: none), 2: RMS norm,
+ * 0: none (no h).  All arithmetic in fp32; h of type A. */
+int32_t nvh_residual_norm(const void* a, int64_t a_stride, const void* a_weight, const void* b, int64_t b_stride, const void* b_weight,
+                          float branch_scale, float branch_eps, const void* c, int64_t c_stride, const float* c32, int64_t c32_stride,
+                          float* x, int32_t norm_kind, const void* norm_weight, const void* norm_bias, float eps, void* h, int64_t h_stride,
+                          int64_t rows, int64_t dim, int32_t act_f32, nvh_stream_t stream);
+/* y[rows, inter] = act(x[:, :inter]) (* x[:, inter:2 inter] when gated), evaluated in fp32.  act 0: silu, 1: gelu (tanh form),
+ * 2: squared relu. */
+int32_t nvh_act_mul(const void* x, int64_t row_stride, void* y, int64_t y_stride, int64_t rows, int64_t inter, int32_t act, int32_t gated,
+                    int32_t act_f32, nvh_stream_t stream);
+/* out fp32 [rows, vocab] = scale * logits, softcapped when cap > 0. */
+int32_t nvh_logits_scale(const void* logits, int64_t row_stride, float* out, int64_t rows, int64_t vocab, float scale, float cap,
+                         int32_t act_f32, nvh_stream_t stream);
+
+/* Linear recurrences with a diagonal decay, state [slots, H, dk, dv] fp32:  S <- diag(w) S + (c k) v^T,  o = S^T q + d v.
+ * nvh_gated_linear_scan: operands fp32; q, k [T, qk_groups, dk] (head h reads group h / (H / qk_groups)), w [T, H, dk] or
+ * [T, H] (w_scalar), kscale = c [T, H] (NULL: 1), v [T, H, dv], skip = d [H] (NULL: 0); strides are per token.  Sequences,
+ * slots and the fresh start as in nvh_delta_scan; out fp32 [T, H dv].  dk <= 256.
+ * nvh_hgrn2_prep: q = silu(q), w = f = lower + (1 - lower) sigmoid(f + f_bias), k = 1 - f, v.
+ * nvh_gla_prep: q * q_scale, k, v, w = sigmoid(decay_logits)^(1 / tau) (decay_logits fp32).
+ * nvh_ssd_conv_prep: the causal convolution (weights [C, taps], last tap on the current token; bias NULL: none) over the
+ * C = inner + 2 gn channels x | B | C of every token, continued from the sequence's carried inputs conv_state
+ * [slots, taps - 1, C] (zeros at a sequence's start), then silu -> out_x [T, inner], out_b, out_c [T, gn];
+ * out_dt = softplus(dt + dt_bias) and out_decay = exp(-exp(a_log) out_dt), both [T, H].
+ * nvh_conv_state_update (after nvh_ssd_conv_prep of the same step): the last taps - 1 inputs of every sequence -> its slot.
+ * nvh_group_rmsnorm_gate: y (type A) = unit over groups of group_size columns of o (o * gate first when gate_first),
+ * times weight ([group_size] shared, or [groups group_size] when weight_full), times gate afterwards otherwise;
+ * gate_act 0: no gate, 1: sigmoid(gate), 2: silu(gate). */
+int32_t nvh_gated_linear_scan(const float* q, int64_t q_stride, const float* k, int64_t k_stride, int64_t qk_groups, const float* w,
+                              int64_t w_stride, int32_t w_scalar, const float* kscale, int64_t kscale_stride, const float* v,
+                              int64_t v_stride, const float* skip, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                              const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
+                              nvh_stream_t stream);
+int32_t nvh_hgrn2_prep(const void* q, int64_t q_stride, const void* f, int64_t f_stride, const void* v, int64_t v_stride,
+                       const void* f_bias, const void* lower, float* out_q, float* out_k, float* out_w, float* out_v,
+                       int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_gla_prep(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                     const float* decay_logits, int64_t z_stride, float q_scale, float tau, float* out_q, float* out_k,
+                     float* out_w, float* out_v, int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_ssd_conv_prep(const void* xbc, int64_t xbc_stride, const void* dt, int64_t dt_stride, const void* conv_w, const void* conv_b,
+                          const void* dt_bias, const void* a_log, float* conv_state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                          const int32_t* context_lens, int64_t batch, int64_t num_tokens, int64_t taps, int64_t heads, int64_t inner,
+                          int64_t gn, float* out_x, float* out_b, float* out_c, float* out_dt, float* out_decay, int32_t act_f32,
+                          nvh_stream_t stream);
+int32_t nvh_conv_state_update(const void* xbc, int64_t xbc_stride, float* conv_state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                              const int32_t* context_lens, int64_t batch, int64_t taps, int64_t channels, int32_t act_f32, nvh_stream_t stream);
+int32_t nvh_group_rmsnorm_gate(const float* o, const void* weight, int32_t weight_full, const void* gate, int64_t gate_stride,
+                               int32_t gate_act, int32_t gate_first, void* y, int64_t y_stride, int64_t rows, int64_t groups,
+                               int64_t group_size, float eps, int32_t act_f32, nvh_stream_t stream);
+
+/* Mixture of experts.  nvh_moe_route: fp32 logits [T, E] -> the `top` largest per token (ties: lower id) as ids [T, top] and
+ * weights [T, top] = softmax restricted to the selected logits.  nvh_moe_align: orders the T top (token, choice) pairs by expert:
+ * src_token[pos] = the pair's token, pos_of_pair[pair] = its position, and tiles of up to 64 positions of one expert
+ * (tile_expert, tile_row0, tile_rows; unused tiles have 0 rows); max_tiles >= nvh_moe_max_tiles(T top, E).
+ * nvh_gemm_grouped_any_nt: y[pos] = x[gather ? gather[pos] : pos] w[expert]^T over the tiles, w [E, N, K]; types as
+ * nvh_gemm_any_nt.  nvh_moe_combine: out fp32 [T, dim] = sum_r weights[t, r] y[pos_of_pair[t, r]] (+ shared[t], type A). */
+int32_t nvh_moe_route(const float* logits, int64_t row_stride, int32_t* ids, float* weights, int64_t num_tokens, int64_t experts,
+                      int64_t top, nvh_stream_t stream);
+int64_t nvh_moe_max_tiles(int64_t pairs, int64_t experts);
+int32_t nvh_moe_align(const int32_t* ids, int64_t num_tokens, int64_t experts, int64_t top, int32_t* src_token, int32_t* pos_of_pair,
+                      int32_t* tile_expert, int32_t* tile_row0, int32_t* tile_rows, int64_t max_tiles, nvh_stream_t stream);
+int32_t nvh_gemm_grouped_any_nt(const void* x, int64_t x_row_stride, const int32_t* gather, const void* w, void* y, int64_t y_row_stride,
+                                const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* tile_rows, int64_t max_tiles,
+                                int64_t N, int64_t K, int32_t in_f32, int32_t out_f32, nvh_stream_t stream);
+int32_t nvh_moe_combine(const void* y, int64_t y_row_stride, const int32_t* pos_of_pair, const float* weights, const void* shared,
+                        int64_t shared_stride, float* out, int64_t num_tokens, int64_t dim, int64_t top, int32_t act_f32, nvh_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -9,6 +9,9 @@
 //                         product wants V^T) and never transposes on the fly.
 //   nvh_attn_paged_any    softmax attention of var-len queries over the paged cache, scores / weights in fp32; the
 //                         epilogue turns each head's output back by the query's position and multiplies the gate.
+//                         Optional: a distance bias, score -= slope[head] * (query position - key position), and a
+//                         sliding window that keeps the first tokens: query i sees key j <= i when i - j < window or
+//                         j < keep_first; key tiles that no query of a workgroup can see are never loaded.
 // Activations and caches are of type A (bf16 or fp32).  Key tiles always start at key 0 of a sequence and every query
 // row keeps its own running maximum and sum, so a query's result does not depend on how the prompt was cut into steps
 // or on what else is in the batch.
@@ -93,18 +96,21 @@ __global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
     const A* qr = row;
     const A* kr = row + nq;
     const A* vr = kr + nk;
-    float sq = 0.f, sk = 0.f;
-    for (int i = threadIdx.x; i < nq; i += 256) {
-        const float v = ldf(qr, i);
-        sq += v * v;
+    float inv_q = 1.f, inv_k = 1.f;
+    if (a.q_norm) {                                          // (null norm weights: q and k pass as they are)
+        float sq = 0.f, sk = 0.f;
+        for (int i = threadIdx.x; i < nq; i += 256) {
+            const float v = ldf(qr, i);
+            sq += v * v;
+        }
+        for (int i = threadIdx.x; i < nk; i += 256) {
+            const float v = ldf(kr, i);
+            sk += v * v;
+        }
+        sq = block_sum_256(sq, red);
+        sk = block_sum_256(sk, red);
+        inv_q = 1.0f / sqrtf(sq / (float)nq + a.eps), inv_k = 1.0f / sqrtf(sk / (float)nk + a.eps);
     }
-    for (int i = threadIdx.x; i < nk; i += 256) {
-        const float v = ldf(kr, i);
-        sk += v * v;
-    }
-    sq = block_sum_256(sq, red);
-    sk = block_sum_256(sk, red);
-    const float inv_q = 1.0f / sqrtf(sq / (float)nq + a.eps), inv_k = 1.0f / sqrtf(sk / (float)nk + a.eps);
     const float pos = (float)a.positions[t];
     const int64_t slot = a.slot_mapping ? a.slot_mapping[t] : -1;
     // q and k: norm, then rotary on the first rot_dims dimensions of every head
@@ -117,13 +123,13 @@ __global__ __launch_bounds__(256) void attn_rotary_prep_kernel(PrepArgs a) {
         if (!dst) continue;
         for (int i = threadIdx.x; i < n; i += 256) {
             const int d = i % a.dim;
-            float v = ldf(src, i) * inv * ldf(wn, i);
+            float v = wn ? ldf(src, i) * inv * ldf(wn, i) : ldf(src, i);
             if (d < a.rot_dims) {
                 int partner, pair;
                 bool first;
                 pair_of(d, a.rot_dims, a.qk_interleaved, partner, pair, first);
                 const int j = i - d + partner;
-                const float o = ldf(src, j) * inv * ldf(wn, j);
+                const float o = wn ? ldf(src, j) * inv * ldf(wn, j) : ldf(src, j);
                 float sn, cs;
                 rot_sincos<A>(pos * a.qk_freq[pair], sn, cs);
                 const float c = cs * a.qk_mag, s = sn * a.qk_mag;
@@ -172,9 +178,30 @@ struct AttnArgs {
     const float* v_freq;       // [vdim/2] or null: no turning back
     int v_interleaved;
     void* out;                 // [T, H*vdim]
+    const float* slopes;       // [H] or null: score -= slopes[head] * (query position - key position)
+    int window, keep_first;    // window > 0: key j is visible to query i only when i - j < window or j < keep_first
     int pages_offset;          // byte offset in LDS of the sequence's page ids (matrix-core kernel)
     int ml_offset;             // ... and of the waves' (max, sum) pairs in the one-query form
 };
+
+// The key tiles (of `tile` keys, starting at multiples of it) that a workgroup whose first query sits at position qlo has to
+// walk: all of them without a window; with one, the tiles that hold kept first tokens and then those from the window of
+// the first query on.  next(k0) is the start of the tile after k0.
+struct TileWalk {
+    int first_end, win_start, tile;
+    __device__ __forceinline__ TileWalk(int window, int keep_first, int qlo, int tile_) : tile(tile_) {
+        first_end = window > 0 ? ((keep_first + tile_ - 1) / tile_) * tile_ : 0;
+        win_start = window > 0 ? (max(qlo - window + 1, 0) / tile_) * tile_ : 0;
+    }
+    __device__ __forceinline__ int next(int k0) const {
+        const int n = k0 + tile;
+        return (n >= first_end && n < win_start) ? win_start : n;
+    }
+};
+
+__device__ __forceinline__ bool key_visible(int key, int qpos, int window, int keep_first) {
+    return key <= qpos && (window <= 0 || qpos - key < window || key < keep_first);
+}
 
 template <typename A>
 __global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
@@ -219,7 +246,9 @@ __global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
     const int qpos = past + q0 + qi;                         // this lane's query position (valid for qi < nq)
     const int last_key = past + q0 + nq - 1;                 // the tile's last query sees keys 0..last_key
     const int32_t* table = a.block_tables + (int64_t)seq * a.table_stride;
-    for (int k0 = 0; k0 <= last_key; k0 += AK) {
+    const float slope = a.slopes ? a.slopes[head] : 0.f;
+    const TileWalk walk(a.window, a.keep_first, past + q0, AK);
+    for (int k0 = walk.first_end > 0 || walk.win_start == 0 ? 0 : walk.win_start; k0 <= last_key; k0 = walk.next(k0)) {
         __syncthreads();                                     // the previous tile's readers are done
         for (int i = tid; i < AK * dim; i += 256) {
             const int r = i / dim, d = i - r * dim, key = k0 + r;
@@ -248,9 +277,9 @@ __global__ __launch_bounds__(256) void attn_paged_any_kernel(AttnArgs a) {
             s0 = __builtin_fmaf(qv, kr0[d], s0);
             s1 = __builtin_fmaf(qv, kr1[d], s1);
         }
-        const bool ok0 = qi < nq && k0 + sub <= qpos, ok1 = qi < nq && k0 + sub + 16 <= qpos;
-        s0 = ok0 ? s0 : -INFINITY;
-        s1 = ok1 ? s1 : -INFINITY;
+        const bool ok0 = qi < nq && key_visible(k0 + sub, qpos, a.window, a.keep_first), ok1 = qi < nq && key_visible(k0 + sub + 16, qpos, a.window, a.keep_first);
+        s0 = ok0 ? s0 - slope * (float)(qpos - (k0 + sub)) : -INFINITY;
+        s1 = ok1 ? s1 - slope * (float)(qpos - (k0 + sub + 16)) : -INFINITY;
         const float m_new = fmaxf(m_run, row16_max(fmaxf(s0, s1)));
         // a row that sees nothing yet keeps m = -inf (only rows past nq: every real query sees key 0)
         const float p0 = ok0 ? expf(s0 - m_new) : 0.f, p1 = ok1 ? expf(s1 - m_new) : 0.f;
@@ -411,11 +440,14 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
             vpre[j] = *reinterpret_cast<const bf16x8*>((const bf16*)a.v_cache + (vbase + c) * a.page + k0 % a.page + piece);
         }
     };
-    // Two register sets, two tiles ahead: the loads of tile t + 2 are issued when tile t has been handed to LDS.
+    // Two register sets, two tiles ahead: the loads of the tile after next are issued when a tile has been handed to LDS.
+    const float slope = a.slopes ? a.slopes[head] : 0.f;
+    const TileWalk walk(a.window, a.keep_first, GROUPED ? past : past + q0, MK);
     bf16x8 kA[KCH], vA[VCH], kB[KCH], vB[VCH];
-    fetch(0, kA, vA);
-    if (MK <= last_key) fetch(MK, kB, vB);
-    auto tile = [&](int k0, bf16x8 (&kpre)[KCH], bf16x8 (&vpre)[VCH]) {
+    int ka = walk.first_end > 0 || walk.win_start == 0 ? 0 : walk.win_start, kb = walk.next(ka);
+    fetch(ka, kA, vA);
+    if (kb <= last_key) fetch(kb, kB, vB);
+    auto tile = [&](int k0, int k_after, bf16x8 (&kpre)[KCH], bf16x8 (&vpre)[VCH]) {
         __syncthreads();
 #pragma unroll
         for (int j = 0; j < KCH; ++j) {
@@ -440,7 +472,7 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
             }
         }
         __syncthreads();
-        if (k0 + 2 * MK <= last_key) fetch(k0 + 2 * MK, kpre, vpre);
+        if (k_after <= last_key) fetch(k_after, kpre, vpre);
         if (wave_idle || k0 > wave_last) return;             // (wave-uniform; the barriers above are passed by all)
         f32x4 sc[NKT];
 #pragma unroll
@@ -460,8 +492,9 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
         for (int t = 0; t < NKT; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
-                const bool ok = qok && k0 + (SPLIT ? wave : t) * 16 + fq * 4 + r <= qpos;
-                sc[t][r] = ok ? sc[t][r] * a.scale : -INFINITY;
+                const int key = k0 + (SPLIT ? wave : t) * 16 + fq * 4 + r;
+                const bool ok = qok && key_visible(key, qpos, a.window, a.keep_first);
+                sc[t][r] = ok ? sc[t][r] * a.scale - slope * (float)(qpos - key) : -INFINITY;
                 mx = fmaxf(mx, sc[t][r]);
             }
         mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
@@ -500,9 +533,14 @@ __global__ __launch_bounds__(256) void attn_paged_mfma_kernel(AttnArgs a) {
                 o[i] = acc;
             }
     };
-    for (int k0 = 0; k0 <= last_key; k0 += 2 * MK) {
-        tile(k0, kA, vA);
-        if (k0 + MK <= last_key) tile(k0 + MK, kB, vB);
+    while (ka <= last_key) {
+        const int ka2 = walk.next(kb);
+        tile(ka, ka2, kA, vA);
+        if (kb > last_key) break;
+        const int kb2 = walk.next(ka2);
+        tile(kb, kb2, kB, vB);
+        ka = ka2;
+        kb = kb2;
     }
     // epilogue through LDS: [MQ][vdim] fp32, then turn back by the query's position, gate, store
     __syncthreads();
@@ -607,7 +645,7 @@ extern "C" int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_strid
                                         void* k_cache, void* v_cache, const int32_t* slot_mapping, int64_t page, int64_t num_tokens,
                                         int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim, int32_t act_f32,
                                         nvh_stream_t stream) {
-    NVH_REQUIRE(proj && q_norm_weight && k_norm_weight && positions && q_out, NVH_EINVAL, "nvh_attn_rotary_prep: null pointer");
+    NVH_REQUIRE(proj && positions && q_out && !q_norm_weight == !k_norm_weight, NVH_EINVAL, "nvh_attn_rotary_prep: null pointer");
     NVH_REQUIRE(num_q_heads > 0 && num_kv_heads > 0 && dim > 0 && vdim > 0 && num_tokens >= 0 && page > 0, NVH_EINVAL, "nvh_attn_rotary_prep: bad sizes");
     NVH_REQUIRE(rot_dims >= 0 && rot_dims <= dim && rot_dims % 2 == 0 && (rot_dims == 0 || qk_freq), NVH_EINVAL,
                 "nvh_attn_rotary_prep: rot_dims %ld does not fit dim %ld", (long)rot_dims, (long)dim);
@@ -627,8 +665,9 @@ extern "C" int32_t nvh_attn_rotary_prep(const void* proj, int64_t proj_row_strid
 extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const void* v_cache, const int32_t* cu_seqlens_q,
                                       const int32_t* context_lens, const int32_t* block_tables, int64_t table_stride, int64_t batch,
                                       int64_t total_q, int64_t page, int64_t num_q_heads, int64_t num_kv_heads, int64_t dim, int64_t vdim,
-                                      float scale, const float* gate, const float* v_freq, int32_t v_interleaved, void* out,
-                                      int32_t act_f32, nvh_stream_t stream) {
+                                      float scale, const float* gate, const float* v_freq, int32_t v_interleaved, const float* slopes,
+                                      int64_t window, int64_t keep_first, void* out, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(window >= 0 && keep_first >= 0 && window < (1 << 30) && keep_first < (1 << 30), NVH_EINVAL, "nvh_attn_paged_any: bad window");
     NVH_REQUIRE(q && k_cache && v_cache && context_lens && block_tables && out, NVH_EINVAL, "nvh_attn_paged_any: null pointer");
     NVH_REQUIRE(batch >= 0 && total_q >= 0 && page > 0 && num_q_heads > 0 && num_kv_heads > 0 && num_q_heads % num_kv_heads == 0 && dim > 0 && vdim > 0,
                 NVH_EINVAL, "nvh_attn_paged_any: bad sizes");
@@ -643,7 +682,7 @@ extern "C" int32_t nvh_attn_paged_any(const void* q, const void* k_cache, const 
     }
     if (batch == 0 || total_q == 0) return NVH_OK;
     AttnArgs a{q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, table_stride, (int)batch, (int)page, (int)num_q_heads,
-               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, 0, 0};
+               (int)num_kv_heads, (int)dim, (int)vdim, scale, gate, v_freq, v_interleaved, out, slopes, (int)window, (int)keep_first, 0, 0};
     // at most ceil(len / AQ) tiles per sequence: total_q / AQ + batch bounds their number (surplus workgroups exit)
     const dim3 grid((unsigned)(total_q / AQ + batch), (unsigned)num_q_heads);
     hipStream_t st = (hipStream_t)stream;

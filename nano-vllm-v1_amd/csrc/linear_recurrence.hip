@@ -1,0 +1,442 @@
+// Linear recurrences with a diagonal decay: a per-head matrix state S [dk, dv] in fp32 that every token updates,
+//   S <- diag(w) S + (c k) v^T,   o = S^T q  (+ d v),
+// with a decay w per key channel (or one per head), a write strength c per head and token, and a skip weight d per head.
+// Gated linear attention (w = a learned decay, c = 1), HGRN2 (w = f, k = 1 - f) and the state-space-duality layer of
+// Mamba-2 (w = exp(-exp(A_log) dt) per head, c = dt, k = B, q = C, v = x, d = D; B and C shared by the heads of a group)
+// are all this one scan; what differs is how the operands are made from the projections:
+//   nvh_hgrn2_prep / nvh_gla_prep / nvh_ssd_conv_prep   projection rows (type A) -> fp32 operands; the last also runs the
+//                    short causal convolution over [x | B | C] with the sequence's carried inputs, silu, softplus of dt
+//   nvh_conv_state_update   leaves the last taps-1 convolution inputs of every sequence in its state slot
+//   nvh_gated_linear_scan   the recurrence: state columns spread over (sequence, head, column block), each column held by
+//                    16 lanes (4 when dk is no multiple of 16) in registers, operands staged through LDS a stage ahead.
+//                    The order of every sum is fixed by the sizes alone: one piece, portions or single tokens give the
+//                    same bits.
+//   nvh_group_rmsnorm_gate  read-out: RMS norm over groups of columns, weight, and a silu / sigmoid gate before or after.
+// Everything that enters the recurrence is fp32; A (bf16 or fp32) is the type of projections, weights and results.
+#include "common.h"
+
+namespace {
+
+template <typename A>
+__device__ __forceinline__ float ldf(const A* p, int64_t i) {
+    return (float)p[i];
+}
+__device__ __forceinline__ float sigmoid_(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float silu_(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float softplus_(float x) { return x > 20.f ? x : log1pf(expf(x)); }
+__device__ __forceinline__ float logsigmoid_(float x) { return fminf(x, 0.f) - log1pf(expf(-fabsf(x))); }
+
+// The sequence that owns packed token t (cu: [batch + 1] ascending; null: token t is sequence t).
+__device__ __forceinline__ int seq_of_token(const int32_t* cu, int batch, int64_t t) {
+    if (!cu) return (int)t;
+    int lo = 0, hi = batch - 1;
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (cu[mid] <= t) lo = mid;
+        else hi = mid - 1;
+    }
+    return lo;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+struct Hgrn2PrepArgs {
+    const void *q, *f, *v;     // projection columns [T, H dk], [T, H dk], [T, H dv]
+    int64_t q_stride, f_stride, v_stride;
+    const void *f_bias, *lower;     // [H dk]
+    float *oq, *ok, *ow, *ov;  // fp32 [T, H dk] x 3, [T, H dv]
+    int64_t n_k, n_v;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void hgrn2_prep_kernel(Hgrn2PrepArgs p) {
+    const int64_t t = blockIdx.x;
+    for (int64_t i = threadIdx.x; i < p.n_k; i += 256) {
+        const float lo = ldf((const A*)p.lower, i);
+        const float f = lo + (1.0f - lo) * sigmoid_(ldf((const A*)p.f, t * p.f_stride + i) + ldf((const A*)p.f_bias, i));
+        p.oq[t * p.n_k + i] = silu_(ldf((const A*)p.q, t * p.q_stride + i));
+        p.ow[t * p.n_k + i] = f;
+        p.ok[t * p.n_k + i] = 1.0f - f;
+    }
+    for (int64_t i = threadIdx.x; i < p.n_v; i += 256) p.ov[t * p.n_v + i] = ldf((const A*)p.v, t * p.v_stride + i);
+}
+
+struct GlaPrepArgs {
+    const void *q, *k, *v;     // projection columns
+    int64_t q_stride, k_stride, v_stride;
+    const float* z;            // fp32 decay logits [T, H dk]
+    int64_t z_stride;
+    float q_scale, inv_tau;
+    float *oq, *ok, *ow, *ov;
+    int64_t n_k, n_v;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void gla_prep_kernel(GlaPrepArgs p) {
+    const int64_t t = blockIdx.x;
+    for (int64_t i = threadIdx.x; i < p.n_k; i += 256) {
+        p.oq[t * p.n_k + i] = ldf((const A*)p.q, t * p.q_stride + i) * p.q_scale;
+        p.ok[t * p.n_k + i] = ldf((const A*)p.k, t * p.k_stride + i);
+        p.ow[t * p.n_k + i] = expf(logsigmoid_(p.z[t * p.z_stride + i]) * p.inv_tau);      // sigmoid(z)^(1/tau)
+    }
+    for (int64_t i = threadIdx.x; i < p.n_v; i += 256) p.ov[t * p.n_v + i] = ldf((const A*)p.v, t * p.v_stride + i);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+struct SsdPrepArgs {
+    const void* xbc;           // [T, ld]: the convolved channels of the in-projection row: x (H dv wide), then B and C (G N wide each)
+    int64_t xbc_stride;
+    const void* dt;            // [T, ld]: H columns
+    int64_t dt_stride;
+    const void *conv_w, *conv_b;    // [C, taps], [C] (null: no bias)
+    const void *dt_bias, *a_log;    // [H]
+    float* conv_state;         // [slots, taps - 1, C]: the inputs of the sequence's last taps - 1 tokens, oldest first
+    const int32_t *slots, *cu_seqlens_q, *context_lens;
+    int batch, taps, H, inner, gn;  // inner = H dv, gn = G N; C = inner + 2 gn
+    float *ov, *ok, *oq, *oc, *ow;  // fp32 [T, inner], [T, gn] (B), [T, gn] (C), [T, H] (dt), [T, H] (decay)
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void ssd_conv_prep_kernel(SsdPrepArgs p) {
+    const int64_t t = blockIdx.x;
+    const int seq = seq_of_token(p.cu_seqlens_q, p.batch, t);
+    const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
+    const int j = (int)t - lo;                               // index of the token among this step's tokens of its sequence
+    const int slot = p.slots[seq];
+    const bool carried = slot >= 0 && p.context_lens[seq] != hi - lo;       // inputs from before this step exist
+    const int C = p.inner + 2 * p.gn, taps = p.taps;
+    const float* st = carried ? p.conv_state + (int64_t)slot * (taps - 1) * C : nullptr;
+    for (int c = threadIdx.x; c < C; c += 256) {
+        float acc = p.conv_b ? ldf((const A*)p.conv_b, c) : 0.f;
+        for (int k = 0; k < taps; ++k) {                     // tap k multiplies the input taps - 1 - k tokens back
+            const int back = taps - 1 - k, src = j - back;
+            float in = 0.f;
+            if (src >= 0) in = ldf((const A*)p.xbc, (t - back) * p.xbc_stride + c);
+            else if (st) in = st[(int64_t)(taps - 1 + src) * C + c];
+            acc = __builtin_fmaf(ldf((const A*)p.conv_w, (int64_t)c * taps + k), in, acc);
+        }
+        const float y = silu_(acc);
+        if (c < p.inner) p.ov[t * p.inner + c] = y;
+        else if (c < p.inner + p.gn) p.ok[t * p.gn + (c - p.inner)] = y;
+        else p.oq[t * p.gn + (c - p.inner - p.gn)] = y;
+    }
+    for (int h = threadIdx.x; h < p.H; h += 256) {
+        const float dt = softplus_(ldf((const A*)p.dt, t * p.dt_stride + h) + ldf((const A*)p.dt_bias, h));
+        p.oc[t * p.H + h] = dt;
+        p.ow[t * p.H + h] = expf(-expf(ldf((const A*)p.a_log, h)) * dt);
+    }
+}
+
+// One thread per (sequence, channel): slot s of the new state is input number n + s - (taps - 1) of [carried | this step's].
+// Ascending s only ever reads carried entries at or above the one it writes.
+template <typename A>
+__global__ __launch_bounds__(256) void conv_state_update_kernel(SsdPrepArgs p) {
+    const int seq = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    const int C = p.inner + 2 * p.gn, keep = p.taps - 1;
+    const int slot = p.slots[seq];
+    if (slot < 0 || c >= C) return;
+    const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
+    const int n = hi - lo;
+    if (n <= 0) return;
+    const bool carried = p.context_lens[seq] != n;
+    float* st = p.conv_state + (int64_t)slot * keep * C;
+    for (int s = 0; s < keep; ++s) {
+        const int src = n + s - keep;
+        float v = 0.f;
+        if (src >= 0) v = ldf((const A*)p.xbc, (int64_t)(lo + src) * p.xbc_stride + c);
+        else if (carried) v = st[(int64_t)(s + n) * C + c];
+        st[(int64_t)s * C + c] = v;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+struct ScanArgs {
+    const float *q, *k;        // [T, QG, dk]: head h reads group h / (H / QG)
+    int64_t q_stride, k_stride;
+    int qk_groups;
+    const float* w;            // decay: [T, H, dk], or [T, H] when w_scalar
+    int64_t w_stride;
+    int w_scalar;
+    const float* kscale;       // [T, H] or null (1)
+    int64_t ks_stride;
+    const float* v;            // [T, H, dv]
+    int64_t v_stride;
+    const float* skip;         // [H] or null
+    float* state;              // [slots, H, dk, dv]
+    const int32_t *slots, *cu_seqlens_q, *context_lens;
+    float* out;                // [T, H dv]
+    int H, dk, dv;
+};
+
+// Lanes per state column (SUBS), rows held per lane (DKQ), EXACT: dk == DKQ * SUBS (rows DKQ sub .. DKQ sub + DKQ - 1 per
+// lane, read from LDS in 16-byte pieces; otherwise rows SUBS ii + sub, those beyond dk held as zeros).  A workgroup owns
+// COLS = 256 / SUBS columns of one (sequence, head).  A token's staged row: q (dk) | k (dk) | w (dk) | v (COLS) | c | padding.
+template <int DKQ, int SUBS, bool EXACT>
+__global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
+    constexpr int COLS = 256 / SUBS;
+    constexpr int CH = (3 * DKQ * SUBS + COLS + 4 + 255) / 256;     // loads per lane and token
+    constexpr int TOK = (32 / CH) < 2 ? 2 : (32 / CH);
+    extern __shared__ __attribute__((aligned(16))) float sm[];
+    const int seq = blockIdx.x, head = blockIdx.y;
+    const int dk = p.dk, dv = p.dv, dkq = (dk + SUBS - 1) / SUBS;
+    const int col0 = blockIdx.z * COLS, lcol = threadIdx.x / SUBS, col = col0 + lcol, sub = threadIdx.x % SUBS;
+    const bool live = col < dv;
+    const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
+    const int slot = p.slots[seq];
+    if (slot < 0 || hi <= lo) return;                        // a padded row (uniform over the workgroup)
+    const bool fresh = p.context_lens[seq] == hi - lo;
+    float* sp = p.state + (((int64_t)slot * p.H + head) * dk) * dv;
+    auto row_of = [&](int ii) { return EXACT ? DKQ * sub + ii : SUBS * ii + sub; };
+    float S[DKQ];
+#pragma unroll
+    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && (EXACT || row_of(ii) < dk)) ? sp[(int64_t)row_of(ii) * dv + col] : 0.f;
+    const int rowf = (3 * dk + COLS + 4) & ~3;             // (a multiple of 4 floats: rows stay 16-byte aligned)
+    const int group = head / (p.H / p.qk_groups);
+    const float* qb = p.q + (int64_t)group * dk;
+    const float* kb = p.k + (int64_t)group * dk;
+    const float* wb = p.w + (p.w_scalar ? (int64_t)head : (int64_t)head * dk);
+    const float* vb = p.v + (int64_t)head * dv;
+    const float skip = p.skip ? p.skip[head] : 0.f;
+    float pre[TOK][CH];
+    auto fetch = [&](int t0) {
+#pragma unroll
+        for (int tt = 0; tt < TOK; ++tt) {
+            const int64_t tok = min(t0 + tt, hi - 1);
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int e = min((int)threadIdx.x + 256 * c, rowf - 1);
+                float x;
+                if (e < dk) x = qb[tok * p.q_stride + e];
+                else if (e < 2 * dk) x = kb[tok * p.k_stride + (e - dk)];
+                else if (e < 3 * dk) x = wb[tok * p.w_stride + (p.w_scalar ? 0 : e - 2 * dk)];
+                else if (e < 3 * dk + COLS) x = vb[tok * p.v_stride + min(col0 + e - 3 * dk, dv - 1)];
+                else x = p.kscale ? p.kscale[tok * p.ks_stride + head] : 1.0f;
+                pre[tt][c] = x;
+            }
+        }
+    };
+    fetch(lo);
+    for (int t0 = lo; t0 < hi; t0 += TOK) {
+        const int nt = min(TOK, hi - t0);
+        __syncthreads();                                     // the previous stage's readers are done
+#pragma unroll
+        for (int tt = 0; tt < TOK; ++tt)
+#pragma unroll
+            for (int c = 0; c < CH; ++c) {
+                const int e = threadIdx.x + 256 * c;
+                if (e < rowf) sm[tt * rowf + e] = pre[tt][c];
+            }
+        __syncthreads();
+        if (t0 + TOK < hi) fetch(t0 + TOK);
+        for (int tt = 0; tt < nt; ++tt) {
+            const float* row = sm + tt * rowf;
+            const float xv = row[3 * dk + lcol];
+            const float sv = row[3 * dk + COLS] * xv;
+            float o = 0.f;
+            if constexpr (EXACT && DKQ % 4 == 0) {
+#pragma unroll
+                for (int c4 = 0; c4 < DKQ / 4; ++c4) {
+                    const int i = DKQ * sub + 4 * c4;
+                    const f32x4 vq = *reinterpret_cast<const f32x4*>(row + i), vk = *reinterpret_cast<const f32x4*>(row + dk + i),
+                                vw = *reinterpret_cast<const f32x4*>(row + 2 * dk + i);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float sn = __builtin_fmaf(vw[e], S[4 * c4 + e], vk[e] * sv);
+                        S[4 * c4 + e] = sn;
+                        o = __builtin_fmaf(sn, vq[e], o);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int ii = 0; ii < DKQ; ++ii)
+                    if (EXACT || ii < dkq) {
+                        const int i = row_of(ii);
+                        const bool in = EXACT || i < dk;     // (a row beyond dk: its state stays zero)
+                        const float xq = in ? row[i] : 0.f, xk = in ? row[dk + i] : 0.f, xw = in ? row[2 * dk + i] : 0.f;
+                        const float sn = __builtin_fmaf(xw, S[ii], xk * sv);
+                        S[ii] = sn;
+                        o = __builtin_fmaf(sn, xq, o);
+                    }
+            }
+            if constexpr (SUBS == 16) {
+                o = row16_sum(o);
+            } else {
+                o += NVH_DPP(o, 0xB1);
+                o += NVH_DPP(o, 0x4E);
+            }
+            if (live && sub == 0) p.out[(int64_t)(t0 + tt) * p.H * dv + head * dv + col] = __builtin_fmaf(skip, xv, o);
+        }
+    }
+    if (live) {
+#pragma unroll
+        for (int ii = 0; ii < DKQ; ++ii)
+            if (EXACT || row_of(ii) < dk) sp[(int64_t)row_of(ii) * dv + col] = S[ii];
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// y[t, g, :] = unit(o') w (* gate afterwards), o' = o (* gate beforehand); one wave per (token, group of `gs` columns).
+// weight: [gs] shared by the groups (w_full 0) or [groups gs] (w_full 1).  gate_act: 0 none, 1 sigmoid, 2 silu.
+template <typename A>
+__global__ __launch_bounds__(256) void group_rmsnorm_gate_kernel(const float* __restrict__ o, const A* __restrict__ weight, int w_full, const A* __restrict__ gate,
+                                                                 int64_t gate_stride, int gate_act, int gate_first, A* __restrict__ y, int64_t y_stride,
+                                                                 int64_t rows, int groups, int gs, float eps) {
+    const int64_t item = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= rows * groups) return;
+    const int64_t t = item / groups;
+    const int g = (int)(item - t * groups), lane = threadIdx.x & 63;
+    const float* orow = o + (t * groups + g) * gs;
+    auto gate_of = [&](int i) {
+        const float z = ldf(gate, t * gate_stride + (int64_t)g * gs + i);
+        return gate_act == 1 ? sigmoid_(z) : silu_(z);
+    };
+    const bool pre = gate && gate_act && gate_first, post = gate && gate_act && !gate_first;
+    float ss = 0.f;
+    for (int i = lane; i < gs; i += 64) {
+        const float v = pre ? orow[i] * gate_of(i) : orow[i];
+        ss += v * v;
+    }
+    ss = wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)gs + eps);
+    for (int i = lane; i < gs; i += 64) {
+        float v = pre ? orow[i] * gate_of(i) : orow[i];
+        v = v * inv * ldf(weight, w_full ? (int64_t)g * gs + i : i);
+        if (post) v *= gate_of(i);
+        y[t * y_stride + (int64_t)g * gs + i] = (A)v;
+    }
+}
+
+template <int DKQ, int SUBS, bool EXACT>
+void launch_scan_as(const ScanArgs& p, int64_t batch, hipStream_t st) {
+    constexpr int COLS = 256 / SUBS;
+    constexpr int CH = (3 * DKQ * SUBS + COLS + 4 + 255) / 256;
+    constexpr int TOK = (32 / CH) < 2 ? 2 : (32 / CH);
+    const dim3 grid((unsigned)batch, (unsigned)p.H, (unsigned)nvh_cdiv(p.dv, COLS));
+    const size_t lds = sizeof(float) * (size_t)TOK * ((3 * p.dk + COLS + 4) & ~3);
+    gated_linear_scan_kernel<DKQ, SUBS, EXACT><<<grid, 256, lds, st>>>(p);
+}
+
+}  // namespace
+
+extern "C" int32_t nvh_hgrn2_prep(const void* q, int64_t q_stride, const void* f, int64_t f_stride, const void* v, int64_t v_stride,
+                                  const void* f_bias, const void* lower, float* out_q, float* out_k, float* out_w, float* out_v,
+                                  int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(q && f && v && f_bias && lower && out_q && out_k && out_w && out_v, NVH_EINVAL, "nvh_hgrn2_prep: null pointer");
+    NVH_REQUIRE(num_tokens >= 0 && n_k > 0 && n_v > 0, NVH_EINVAL, "nvh_hgrn2_prep: bad sizes");
+    if (num_tokens == 0) return NVH_OK;
+    const Hgrn2PrepArgs p{q, f, v, q_stride, f_stride, v_stride, f_bias, lower, out_q, out_k, out_w, out_v, n_k, n_v};
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) hgrn2_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
+    else hgrn2_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_hgrn2_prep");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_gla_prep(const void* q, int64_t q_stride, const void* k, int64_t k_stride, const void* v, int64_t v_stride,
+                                const float* decay_logits, int64_t z_stride, float q_scale, float tau, float* out_q, float* out_k,
+                                float* out_w, float* out_v, int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(q && k && v && decay_logits && out_q && out_k && out_w && out_v, NVH_EINVAL, "nvh_gla_prep: null pointer");
+    NVH_REQUIRE(num_tokens >= 0 && n_k > 0 && n_v > 0 && tau > 0.f, NVH_EINVAL, "nvh_gla_prep: bad sizes");
+    if (num_tokens == 0) return NVH_OK;
+    const GlaPrepArgs p{q, k, v, q_stride, k_stride, v_stride, decay_logits, z_stride, q_scale, 1.0f / tau, out_q, out_k, out_w, out_v, n_k, n_v};
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) gla_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
+    else gla_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_gla_prep");
+    return NVH_OK;
+}
+
+static int32_t ssd_args(SsdPrepArgs& p, const void* xbc, int64_t xbc_stride, const void* dt, int64_t dt_stride, const void* conv_w, const void* conv_b,
+                        const void* dt_bias, const void* a_log, float* conv_state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                        const int32_t* context_lens, int64_t batch, int64_t taps, int64_t heads, int64_t inner, int64_t gn) {
+    NVH_REQUIRE(xbc && conv_w && slots && context_lens && (taps == 1 || conv_state), NVH_EINVAL, "ssd convolution: null pointer");
+    NVH_REQUIRE(batch >= 0 && taps >= 1 && taps <= 64 && heads > 0 && inner > 0 && gn > 0 && xbc_stride >= inner + 2 * gn, NVH_EINVAL, "ssd convolution: bad sizes");
+    p = SsdPrepArgs{xbc, xbc_stride, dt, dt_stride, conv_w, conv_b, dt_bias, a_log, conv_state, slots, cu_seqlens_q, context_lens,
+                    (int)batch, (int)taps, (int)heads, (int)inner, (int)gn, nullptr, nullptr, nullptr, nullptr, nullptr};
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_ssd_conv_prep(const void* xbc, int64_t xbc_stride, const void* dt, int64_t dt_stride, const void* conv_w, const void* conv_b,
+                                     const void* dt_bias, const void* a_log, float* conv_state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                                     const int32_t* context_lens, int64_t batch, int64_t num_tokens, int64_t taps, int64_t heads, int64_t inner,
+                                     int64_t gn, float* out_x, float* out_b, float* out_c, float* out_dt, float* out_decay, int32_t act_f32,
+                                     nvh_stream_t stream) {
+    SsdPrepArgs p;
+    const int32_t rc = ssd_args(p, xbc, xbc_stride, dt, dt_stride, conv_w, conv_b, dt_bias, a_log, conv_state, slots, cu_seqlens_q, context_lens, batch, taps, heads, inner, gn);
+    if (rc != NVH_OK) return rc;
+    NVH_REQUIRE(dt && dt_bias && a_log && out_x && out_b && out_c && out_dt && out_decay && num_tokens >= 0, NVH_EINVAL, "nvh_ssd_conv_prep: null pointer");
+    NVH_REQUIRE(cu_seqlens_q || num_tokens == batch, NVH_EINVAL, "nvh_ssd_conv_prep: one token per sequence without cu_seqlens_q");
+    if (num_tokens == 0 || batch == 0) return NVH_OK;
+    p.ov = out_x, p.ok = out_b, p.oq = out_c, p.oc = out_dt, p.ow = out_decay;
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) ssd_conv_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
+    else ssd_conv_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_ssd_conv_prep");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_conv_state_update(const void* xbc, int64_t xbc_stride, float* conv_state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                                         const int32_t* context_lens, int64_t batch, int64_t taps, int64_t channels, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(xbc && slots && context_lens && batch >= 0 && taps >= 1 && channels > 0 && xbc_stride >= channels, NVH_EINVAL, "nvh_conv_state_update: bad argument");
+    if (batch == 0 || taps == 1) return NVH_OK;
+    NVH_REQUIRE(conv_state, NVH_EINVAL, "nvh_conv_state_update: null state");
+    SsdPrepArgs p{};
+    p.xbc = xbc, p.xbc_stride = xbc_stride, p.conv_state = conv_state, p.slots = slots, p.cu_seqlens_q = cu_seqlens_q, p.context_lens = context_lens;
+    p.batch = (int)batch, p.taps = (int)taps, p.inner = (int)channels, p.gn = 0;
+    hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((unsigned)batch, (unsigned)nvh_cdiv(channels, 256));
+    if (act_f32) conv_state_update_kernel<float><<<grid, 256, 0, st>>>(p);
+    else conv_state_update_kernel<bf16><<<grid, 256, 0, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_conv_state_update");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_gated_linear_scan(const float* q, int64_t q_stride, const float* k, int64_t k_stride, int64_t qk_groups, const float* w,
+                                         int64_t w_stride, int32_t w_scalar, const float* kscale, int64_t kscale_stride, const float* v,
+                                         int64_t v_stride, const float* skip, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
+                                         const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
+                                         nvh_stream_t stream) {
+    NVH_REQUIRE(q && k && w && v && state && slots && context_lens && out, NVH_EINVAL, "nvh_gated_linear_scan: null pointer");
+    NVH_REQUIRE(batch >= 0 && heads > 0 && dk > 0 && dv > 0 && qk_groups > 0 && heads % qk_groups == 0, NVH_EINVAL, "nvh_gated_linear_scan: bad sizes");
+    NVH_REQUIRE(dk <= 256, NVH_ENOSYS, "nvh_gated_linear_scan: key size %ld above 256", (long)dk);
+    if (batch == 0) return NVH_OK;
+    const ScanArgs p{q, k, q_stride, k_stride, (int)qk_groups, w, w_stride, w_scalar, kscale, kscale_stride, v, v_stride, skip, state, slots,
+                     cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dv};
+    hipStream_t st = (hipStream_t)stream;
+    // (the choice depends on dk alone, so a sequence sees one summation order whatever the batch or the cut)
+    if (dk % 16 == 0) {
+        switch (dk / 16) {
+            case 1: launch_scan_as<1, 16, true>(p, batch, st); break;
+            case 2: launch_scan_as<2, 16, true>(p, batch, st); break;
+            case 3: launch_scan_as<3, 16, true>(p, batch, st); break;
+            case 4: launch_scan_as<4, 16, true>(p, batch, st); break;
+            case 6: launch_scan_as<6, 16, true>(p, batch, st); break;
+            case 8: launch_scan_as<8, 16, true>(p, batch, st); break;
+            case 16: launch_scan_as<16, 16, true>(p, batch, st); break;
+            default:
+                if (dk / 16 <= 8) launch_scan_as<8, 16, false>(p, batch, st);
+                else launch_scan_as<16, 16, false>(p, batch, st);
+        }
+    } else {
+        const int dkq = (int)(dk + 3) / 4;
+        if (dkq <= 8) launch_scan_as<8, 4, false>(p, batch, st);
+        else if (dkq <= 16) launch_scan_as<16, 4, false>(p, batch, st);
+        else if (dkq <= 32) launch_scan_as<32, 4, false>(p, batch, st);
+        else launch_scan_as<64, 4, false>(p, batch, st);
+    }
+    NVH_CHECK_LAUNCH("nvh_gated_linear_scan");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_group_rmsnorm_gate(const float* o, const void* weight, int32_t weight_full, const void* gate, int64_t gate_stride,
+                                          int32_t gate_act, int32_t gate_first, void* y, int64_t y_stride, int64_t rows, int64_t groups,
+                                          int64_t group_size, float eps, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(o && weight && y && rows >= 0 && groups > 0 && group_size > 0 && gate_act >= 0 && gate_act <= 2 && (!gate_act || gate), NVH_EINVAL,
+                "nvh_group_rmsnorm_gate: bad argument");
+    if (rows == 0) return NVH_OK;
+    const unsigned blocks = (unsigned)nvh_cdiv(rows * groups, 4);
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) group_rmsnorm_gate_kernel<float><<<dim3(blocks), 256, 0, st>>>(o, (const float*)weight, weight_full, (const float*)gate, gate_stride, gate_act, gate_first, (float*)y, y_stride, rows, (int)groups, (int)group_size, eps);
+    else group_rmsnorm_gate_kernel<bf16><<<dim3(blocks), 256, 0, st>>>(o, (const bf16*)weight, weight_full, (const bf16*)gate, gate_stride, gate_act, gate_first, (bf16*)y, y_stride, rows, (int)groups, (int)group_size, eps);
+    NVH_CHECK_LAUNCH("nvh_group_rmsnorm_gate");
+    return NVH_OK;
+}

@@ -1,0 +1,216 @@
+// Mixture of experts: a token goes to the `top` experts whose router logits are largest, mixed with the weights that a
+// softmax over just these `top` logits gives.
+//   nvh_moe_route     fp32 router logits [T, E] -> expert ids and weights [T, top] (ties go to the lower expert id)
+//   nvh_moe_align     the (token, choice) pairs ordered by expert: for every position in that order the token it comes
+//                     from, for every pair its position, and a list of 64-row tiles (expert, first position, rows) that
+//                     covers every expert's block - all on the device, so a step never waits for the host and the whole
+//                     layer can sit in a captured graph (the tile list has a fixed upper bound: pairs / 64 + experts)
+//   nvh_gemm_grouped_any_nt   y[pos] = x[src(pos)] W[expert of pos]^T over that tile list: the any-shape product
+//                     (gemm_any.h) with a weight matrix per tile and rows gathered through an index, bf16 on the matrix
+//                     cores or true fp32.  A row's result does not depend on where in its expert's block it lies.
+//   nvh_moe_combine   out fp32 [T, dim] = sum over a token's choices, in choice order, of weight * y[pos] (+ shared[t])
+#include "common.h"
+#include "gemm_any.h"
+
+namespace {
+
+// One wave per token: lane l holds logits l, l + 64, ...; `top` rounds of a wave-wide argmax.
+constexpr int ROUTE_MAX_PER_LANE = 16;      // experts <= 1024
+
+__global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict__ logits, int64_t stride, int32_t* __restrict__ ids, float* __restrict__ weights,
+                                                        int64_t tokens, int experts, int top) {
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= tokens) return;
+    const int lane = threadIdx.x & 63;
+    float z[ROUTE_MAX_PER_LANE];
+#pragma unroll
+    for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+        const int e = lane + 64 * j;
+        z[j] = e < experts ? logits[t * stride + e] : -INFINITY;
+    }
+    float first = 0.f, denom = 0.f;
+    for (int r = 0; r < top; ++r) {
+        float bv = -INFINITY;
+        int be = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+            const int e = lane + 64 * j;
+            if (z[j] > bv || (z[j] == bv && e < be && z[j] != -INFINITY)) {
+                bv = z[j];
+                be = e;
+            }
+        }
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oe = __shfl_xor(be, off, 64);
+            if (ov > bv || (ov == bv && oe < be)) {
+                bv = ov;
+                be = oe;
+            }
+        }
+        if (r == 0) first = bv;
+        const float w = expf(bv - first);                    // the first choice is the largest: exponents <= 0
+        denom += w;
+        if (lane == 0) {
+            ids[t * top + r] = be;
+            weights[t * top + r] = w;
+        }
+#pragma unroll
+        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
+            if (lane + 64 * j == be) z[j] = -INFINITY;       // taken
+    }
+    if (lane == 0)
+        for (int r = 0; r < top; ++r) weights[t * top + r] = weights[t * top + r] / denom;
+}
+
+// One workgroup: counts per expert, block starts, then every pair takes the next free position of its expert's block.
+// (Which position a pair gets within its block depends on the order the lanes arrive in; nothing downstream depends on it.)
+__global__ __launch_bounds__(1024) void moe_align_kernel(const int32_t* __restrict__ ids, int64_t pairs, int experts, int top, int32_t* __restrict__ src_token,
+                                                         int32_t* __restrict__ pos_of_pair, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
+                                                         int32_t* __restrict__ tile_rows, int max_tiles) {
+    extern __shared__ int sh[];                              // [experts] counts, [experts] starts / cursors, [experts] first tile
+    int* count = sh;
+    int* start = sh + experts;
+    int* tile0 = sh + 2 * experts;
+    for (int e = threadIdx.x; e < experts; e += 1024) count[e] = 0;
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < pairs; i += 1024) {
+        const int e = ids[i];
+        if (e >= 0 && e < experts) atomicAdd(&count[e], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int row = 0, tile = 0;
+        for (int e = 0; e < experts; ++e) {
+            start[e] = row;
+            tile0[e] = tile;
+            row += count[e];
+            tile += (count[e] + nvh_any::GT - 1) / nvh_any::GT;
+        }
+        tile0[experts] = tile;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < max_tiles; i += 1024) tile_rows[i] = 0;
+    __syncthreads();
+    for (int e = threadIdx.x; e < experts; e += 1024) {
+        const int n = count[e];
+        for (int k = 0, t = tile0[e]; k < n && t < max_tiles; k += nvh_any::GT, ++t) {
+            tile_expert[t] = e;
+            tile_row0[t] = start[e] + k;
+            tile_rows[t] = min(nvh_any::GT, n - k);
+        }
+    }
+    __syncthreads();
+    for (int64_t i = threadIdx.x; i < pairs; i += 1024) {
+        const int e = ids[i];
+        if (e < 0 || e >= experts) {
+            pos_of_pair[i] = -1;
+            continue;
+        }
+        const int pos = atomicAdd(&start[e], 1);
+        src_token[pos] = (int32_t)(i / top);
+        pos_of_pair[i] = pos;
+    }
+}
+
+struct GroupedArgs {
+    const void* x;             // rows of K
+    int64_t ldx;
+    const int32_t* gather;     // [pairs]: source row of x for every output row (null: the output row's own index)
+    const void* w;             // [experts, N, K]
+    void* y;                   // [pairs, N]
+    int64_t ldy;
+    const int32_t *tile_expert, *tile_row0, *tile_rows;
+    int N, K, vec_ok;
+};
+
+template <bool OUT_F32>
+__global__ __launch_bounds__(256) void gemm_grouped_bf16_kernel(GroupedArgs a) {
+    const int rows = a.tile_rows[blockIdx.y];
+    if (rows <= 0) return;                                   // (uniform: a tile beyond the list's end)
+    const bf16* w = (const bf16*)a.w + (int64_t)a.tile_expert[blockIdx.y] * a.N * a.K;
+    nvh_any::gemm_any_bf16_tile<OUT_F32>((const bf16*)a.x, a.ldx, w, a.K, nullptr, a.y, a.ldy, nvh_any::RowMap{a.gather, a.tile_row0[blockIdx.y], rows},
+                                         blockIdx.x * nvh_any::GT, a.N, a.K, a.vec_ok);
+}
+
+__global__ __launch_bounds__(256) void gemm_grouped_f32_kernel(GroupedArgs a) {
+    const int rows = a.tile_rows[blockIdx.y];
+    if (rows <= 0) return;
+    const float* w = (const float*)a.w + (int64_t)a.tile_expert[blockIdx.y] * a.N * a.K;
+    nvh_any::gemm_any_f32_tile((const float*)a.x, a.ldx, w, a.K, nullptr, (float*)a.y, a.ldy, nvh_any::RowMap{a.gather, a.tile_row0[blockIdx.y], rows},
+                               blockIdx.x * nvh_any::GT, a.N, a.K);
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const A* __restrict__ y, int64_t ldy, const int32_t* __restrict__ pos_of_pair, const float* __restrict__ weights,
+                                                          const A* __restrict__ shared, int64_t shared_stride, float* __restrict__ out, int dim, int top) {
+    const int64_t t = blockIdx.x;
+    for (int c = threadIdx.x; c < dim; c += 256) {
+        float s = 0.f;
+        for (int r = 0; r < top; ++r) {
+            const int pos = pos_of_pair[t * top + r];
+            if (pos >= 0) s = __builtin_fmaf(weights[t * top + r], (float)y[(int64_t)pos * ldy + c], s);
+        }
+        if (shared) s += (float)shared[t * shared_stride + c];
+        out[t * dim + c] = s;
+    }
+}
+
+}  // namespace
+
+extern "C" int32_t nvh_moe_route(const float* logits, int64_t row_stride, int32_t* ids, float* weights, int64_t num_tokens, int64_t experts,
+                                 int64_t top, nvh_stream_t stream) {
+    NVH_REQUIRE(logits && ids && weights, NVH_EINVAL, "nvh_moe_route: null pointer");
+    NVH_REQUIRE(num_tokens >= 0 && experts > 0 && top > 0 && top <= experts && row_stride >= experts, NVH_EINVAL, "nvh_moe_route: bad sizes");
+    NVH_REQUIRE(experts <= 64 * ROUTE_MAX_PER_LANE, NVH_ENOSYS, "nvh_moe_route: %ld experts above %d", (long)experts, 64 * ROUTE_MAX_PER_LANE);
+    if (num_tokens == 0) return NVH_OK;
+    moe_route_kernel<<<dim3((unsigned)nvh_cdiv(num_tokens, 4)), 256, 0, (hipStream_t)stream>>>(logits, row_stride, ids, weights, num_tokens, (int)experts, (int)top);
+    NVH_CHECK_LAUNCH("nvh_moe_route");
+    return NVH_OK;
+}
+
+extern "C" int64_t nvh_moe_max_tiles(int64_t pairs, int64_t experts) { return pairs / nvh_any::GT + experts; }
+
+extern "C" int32_t nvh_moe_align(const int32_t* ids, int64_t num_tokens, int64_t experts, int64_t top, int32_t* src_token, int32_t* pos_of_pair,
+                                 int32_t* tile_expert, int32_t* tile_row0, int32_t* tile_rows, int64_t max_tiles, nvh_stream_t stream) {
+    NVH_REQUIRE(ids && src_token && pos_of_pair && tile_expert && tile_row0 && tile_rows, NVH_EINVAL, "nvh_moe_align: null pointer");
+    NVH_REQUIRE(num_tokens >= 0 && experts > 0 && experts <= 4096 && top > 0 && max_tiles >= nvh_moe_max_tiles(num_tokens * top, experts) && num_tokens * top < (1 << 30),
+                NVH_EINVAL, "nvh_moe_align: bad sizes");
+    if (num_tokens == 0) return NVH_OK;
+    const size_t lds = sizeof(int) * (size_t)(3 * experts + 1);
+    moe_align_kernel<<<dim3(1), 1024, lds, (hipStream_t)stream>>>(ids, num_tokens * top, (int)experts, (int)top, src_token, pos_of_pair, tile_expert, tile_row0,
+                                                                  tile_rows, (int)max_tiles);
+    NVH_CHECK_LAUNCH("nvh_moe_align");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_gemm_grouped_any_nt(const void* x, int64_t x_row_stride, const int32_t* gather, const void* w, void* y, int64_t y_row_stride,
+                                           const int32_t* tile_expert, const int32_t* tile_row0, const int32_t* tile_rows, int64_t max_tiles,
+                                           int64_t N, int64_t K, int32_t in_f32, int32_t out_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(x && w && y && tile_expert && tile_row0 && tile_rows, NVH_EINVAL, "nvh_gemm_grouped_any_nt: null pointer");
+    NVH_REQUIRE(max_tiles >= 0 && max_tiles < 65536 && N > 0 && K > 0 && N < (1 << 30) && K < (1 << 30) && x_row_stride >= K && y_row_stride >= N, NVH_EINVAL,
+                "nvh_gemm_grouped_any_nt: bad sizes");
+    NVH_REQUIRE(!in_f32 || out_f32, NVH_ENOSYS, "nvh_gemm_grouped_any_nt: fp32 operands give an fp32 product");
+    if (max_tiles == 0) return NVH_OK;
+    const int vec_ok = !in_f32 && K % 8 == 0 && x_row_stride % 8 == 0 && nvh_aligned16(x) && nvh_aligned16(w);
+    const GroupedArgs a{x, x_row_stride, gather, w, y, y_row_stride, tile_expert, tile_row0, tile_rows, (int)N, (int)K, vec_ok};
+    const dim3 grid((unsigned)nvh_cdiv(N, nvh_any::GT), (unsigned)max_tiles);
+    hipStream_t st = (hipStream_t)stream;
+    if (in_f32) gemm_grouped_f32_kernel<<<grid, 256, 0, st>>>(a);
+    else if (out_f32) gemm_grouped_bf16_kernel<true><<<grid, 256, 0, st>>>(a);
+    else gemm_grouped_bf16_kernel<false><<<grid, 256, 0, st>>>(a);
+    NVH_CHECK_LAUNCH("nvh_gemm_grouped_any_nt");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_moe_combine(const void* y, int64_t y_row_stride, const int32_t* pos_of_pair, const float* weights, const void* shared,
+                                   int64_t shared_stride, float* out, int64_t num_tokens, int64_t dim, int64_t top, int32_t act_f32, nvh_stream_t stream) {
+    NVH_REQUIRE(y && pos_of_pair && weights && out && num_tokens >= 0 && dim > 0 && top > 0 && y_row_stride >= dim, NVH_EINVAL, "nvh_moe_combine: bad argument");
+    if (num_tokens == 0) return NVH_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) moe_combine_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>((const float*)y, y_row_stride, pos_of_pair, weights, (const float*)shared, shared_stride, out, (int)dim, (int)top);
+    else moe_combine_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>((const bf16*)y, y_row_stride, pos_of_pair, weights, (const bf16*)shared, shared_stride, out, (int)dim, (int)top);
+    NVH_CHECK_LAUNCH("nvh_moe_combine");
+    return NVH_OK;
+}

@@ -4,6 +4,7 @@
 //   tanh-GELU gate, [stream | first embedding] concatenation for a looped stack, row gather, logit softcap.
 // Every kernel is one workgroup per row (or a flat element grid) with 16-byte accesses where the row allows.
 #include "common.h"
+#include "gemm_any.h"
 
 namespace {
 
@@ -134,124 +135,149 @@ __global__ __launch_bounds__(256) void softcap_kernel(const A* __restrict__ z, i
     out[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
 }
 
-// ---------------------------------------------------------------------------------------------------------------
-// y[M, N] = x[M, K] w[N, K]^T (+ bias[N]) for ANY M, N, K (ragged edges are zero-filled on the way into LDS and masked on
-// the way out).  The order in which an output element sums over k depends on (N, K) only, never on M or on the row's
-// place in the batch.  bf16: 64 x 64 tile per workgroup, four waves of 2 x 2 MFMA 16x16x32 tiles, fp32 accumulation.
-// fp32: the same tile with 4 x 4 outputs per lane on the vector ALU (true fp32 products and sums).
-constexpr int GT = 64, GK = 64, GLD = GK + 8;
+// x[row] = table[id] * scale + pos_table[position] (fp32); ids or positions outside their tables give zeros for that term.
+template <typename A>
+__global__ __launch_bounds__(256) void embedding_pos_stream_kernel(const int64_t* __restrict__ ids, const int64_t* __restrict__ positions,
+                                                                   const A* __restrict__ table, const A* __restrict__ pos_table, float scale,
+                                                                   float* __restrict__ x, int dim, int64_t vocab, int64_t max_pos) {
+    const int64_t row = blockIdx.x;
+    const int64_t id = ids[row], p = pos_table ? positions[row] : -1;
+    const bool ok = id >= 0 && id < vocab, pok = p >= 0 && p < max_pos;
+    for (int c = threadIdx.x; c < dim; c += 256) {
+        const float e = ok ? (float)table[id * dim + c] * scale : 0.f;
+        x[row * dim + c] = e + (pok ? (float)pos_table[p * dim + c] : 0.f);
+    }
+}
 
+__device__ __forceinline__ float block_sum4(float v, float* scratch) {
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return scratch[0] + scratch[1] + scratch[2] + scratch[3];
+}
+
+// The close of a layer whose sublayers all read one norm of the stream, and the norm that opens the next layer, per row:
+//   s = branch_scale * (unit(a) wa + unit(b) wb) + c + c32;   x <- x + s;   h <- norm(x)
+// unit(v) = v / sqrt(mean(v^2) + branch_eps) where the branch has a weight (wa / wb), v itself where it has none; absent
+// terms are skipped.  norm: 1 = layer norm ((x - mean) / sqrt(var + eps) w + b, var the mean squared deviation),
+// 2 = RMS norm (x rsqrt(mean of squares + eps) w), 0 = none (no h).  Everything is fp32; the row sits in LDS meanwhile.
+struct CloseArgs {
+    const void *a, *wa, *b, *wb, *c;
+    const float* c32;
+    int64_t a_stride, b_stride, c_stride, c32_stride;
+    float branch_scale, branch_eps;
+    float* x;
+    int norm;
+    const void *nw, *nb;
+    float eps;
+    void* h;
+    int64_t h_stride;
+    int dim;
+};
+
+template <typename A>
+__global__ __launch_bounds__(256) void residual_norm_kernel(CloseArgs p) {
+    extern __shared__ float rowbuf[];
+    __shared__ float red[4];
+    const int64_t row = blockIdx.x;
+    const int dim = p.dim;
+    const A* a = p.a ? (const A*)p.a + row * p.a_stride : nullptr;
+    const A* b = p.b ? (const A*)p.b + row * p.b_stride : nullptr;
+    const A* c = p.c ? (const A*)p.c + row * p.c_stride : nullptr;
+    const float* c32 = p.c32 ? p.c32 + row * p.c32_stride : nullptr;
+    float ia = 1.f, ib = 1.f;
+    if (a && p.wa) {
+        float s = 0.f;
+        for (int i = threadIdx.x; i < dim; i += 256) {
+            const float v = (float)a[i];
+            s += v * v;
+        }
+        ia = 1.0f / sqrtf(block_sum4(s, red) / (float)dim + p.branch_eps);
+    }
+    if (b && p.wb) {
+        float s = 0.f;
+        for (int i = threadIdx.x; i < dim; i += 256) {
+            const float v = (float)b[i];
+            s += v * v;
+        }
+        ib = 1.0f / sqrtf(block_sum4(s, red) / (float)dim + p.branch_eps);
+    }
+    float* xr = p.x + row * dim;
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        float s = 0.f;
+        if (a) s += p.wa ? (float)a[i] * ia * (float)((const A*)p.wa)[i] : (float)a[i];
+        if (b) s += p.wb ? (float)b[i] * ib * (float)((const A*)p.wb)[i] : (float)b[i];
+        s *= p.branch_scale;
+        if (c) s += (float)c[i];
+        if (c32) s += c32[i];
+        const float v = xr[i] + s;
+        if (a || b || c || c32) xr[i] = v;
+        rowbuf[i] = v;
+        sum += v;
+    }
+    if (p.norm == 0) return;
+    float mean = 0.f;
+    if (p.norm == 1) mean = block_sum4(sum, red) / (float)dim;
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        const float d = rowbuf[i] - mean;
+        sq += d * d;
+    }
+    const float inv = 1.0f / sqrtf(block_sum4(sq, red) / (float)dim + p.eps);
+    A* h = (A*)p.h + row * p.h_stride;
+    for (int i = threadIdx.x; i < dim; i += 256) {
+        float v = (rowbuf[i] - mean) * inv * (float)((const A*)p.nw)[i];
+        if (p.nb) v += (float)((const A*)p.nb)[i];
+        h[i] = (A)v;
+    }
+}
+
+// y = act(g) (* u when gated): g = columns [0, inter) and u = columns [inter, 2 inter) of the row.
+// act: 0 silu, 1 gelu (tanh form), 2 squared relu.
+template <typename A>
+__global__ __launch_bounds__(256) void act_mul_kernel(const A* __restrict__ gu, int64_t gu_stride, A* __restrict__ y, int64_t y_stride, int64_t rows, int inter,
+                                                      int act, int gated) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * inter) return;
+    const int64_t row = i / inter;
+    const int c = (int)(i - row * inter);
+    const float g = ldf(gu, row * gu_stride + c);
+    float v;
+    if (act == 0) v = g / (1.0f + expf(-g));
+    else if (act == 1) v = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    else v = g > 0.f ? g * g : 0.f;
+    if (gated) v *= ldf(gu, row * gu_stride + inter + c);
+    y[row * y_stride + c] = (A)v;
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void logits_scale_kernel(const A* __restrict__ z, int64_t z_stride, float* __restrict__ out, int64_t rows, int vocab, float scale,
+                                                           float cap) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows * vocab) return;
+    const int64_t row = i / vocab;
+    const float v = ldf(z, row * z_stride + (i - row * vocab)) * scale;
+    out[i] = cap > 0.f ? cap * tanhf(v / cap) : v;
+}
+
+
+// ---------------------------------------------------------------------------------------------------------------
+// The any-shape product (gemm_any.h) over one weight matrix: tile (blockIdx.x, blockIdx.y) covers 64 columns and the 64
+// rows that start at 64 blockIdx.y.
 template <bool OUT_F32>
 __global__ __launch_bounds__(256) void gemm_any_bf16_kernel(const bf16* __restrict__ x, int64_t ldx, const bf16* __restrict__ w, int64_t ldw,
                                                             const bf16* __restrict__ bias, void* __restrict__ yv, int64_t ldy, int M, int N, int K,
                                                             int vec_ok) {
-    __shared__ __attribute__((aligned(16))) bf16 xs[GT * GLD];
-    __shared__ __attribute__((aligned(16))) bf16 ws[GT * GLD];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, fr = lane & 15, fq = lane >> 4;
-    const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
-    const int wm = (wave >> 1) * 32, wn = (wave & 1) * 32;
-    f32x4 acc[2][2];
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-    const int lr = tid >> 2, lc = (tid & 3) * 16;            // this thread's row and first column of the 64 x 64 tile
-    for (int k0 = 0; k0 < K; k0 += GK) {
-        // stage both tiles
-#pragma unroll
-        for (int which = 0; which < 2; ++which) {
-            const bf16* src = which ? w : x;
-            const int64_t ld = which ? ldw : ldx;
-            const int row = (which ? n0 : m0) + lr, rows = which ? N : M;
-            bf16* dst = (which ? ws : xs) + lr * GLD + lc;
-#pragma unroll
-            for (int half = 0; half < 2; ++half) {
-                const int kc = k0 + lc + half * 8;
-                bf16x8 v;
-                if (row < rows && vec_ok && kc + 8 <= K) {
-                    v = *reinterpret_cast<const bf16x8*>(src + (int64_t)row * ld + kc);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) v[e] = (row < rows && kc + e < K) ? src[(int64_t)row * ld + kc + e] : (bf16)0.f;
-                }
-                *reinterpret_cast<bf16x8*>(dst + half * 8) = v;
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int ks = 0; ks < GK / 32; ++ks) {
-            bf16x8 wf[2], xf[2];
-#pragma unroll
-            for (int i = 0; i < 2; ++i) {
-                wf[i] = *reinterpret_cast<const bf16x8*>(ws + (wn + i * 16 + fr) * GLD + ks * 32 + fq * 8);
-                xf[i] = *reinterpret_cast<const bf16x8*>(xs + (wm + i * 16 + fr) * GLD + ks * 32 + fq * 8);
-            }
-#pragma unroll
-            for (int i = 0; i < 2; ++i)
-#pragma unroll
-                for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[i], xf[j], acc[i][j], 0, 0, 0);
-        }
-        __syncthreads();
-    }
-    // lane holds, for weight tile i and row tile j: row m = wm + 16 j + fr, columns n = wn + 16 i + 4 fq + e
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int m = m0 + wm + j * 16 + fr;
-            if (m >= M) continue;
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const int n = n0 + wn + i * 16 + fq * 4 + e;
-                if (n >= N) continue;
-                float v = acc[i][j][e];
-                if (bias) v += (float)bias[n];
-                if constexpr (OUT_F32) ((float*)yv)[(int64_t)m * ldy + n] = v;
-                else ((bf16*)yv)[(int64_t)m * ldy + n] = (bf16)v;
-            }
-        }
+    const int m0 = blockIdx.y * nvh_any::GT;
+    nvh_any::gemm_any_bf16_tile<OUT_F32>(x, ldx, w, ldw, bias, yv, ldy, nvh_any::RowMap{nullptr, m0, min(nvh_any::GT, M - m0)}, blockIdx.x * nvh_any::GT, N, K, vec_ok);
 }
 
 __global__ __launch_bounds__(256) void gemm_any_f32_kernel(const float* __restrict__ x, int64_t ldx, const float* __restrict__ w, int64_t ldw,
                                                            const float* __restrict__ bias, float* __restrict__ y, int64_t ldy, int M, int N, int K) {
-    constexpr int BK = 16;
-    __shared__ float xs[BK][GT + 4];
-    __shared__ float ws[BK][GT + 4];
-    const int tid = threadIdx.x;
-    const int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
-    const int tm = (tid >> 4) * 4, tn = (tid & 15) * 4;
-    float acc[4][4] = {};
-    const int lr = tid >> 2, lc = (tid & 3) * 4;             // 64 rows x 16 columns per stage: 4 consecutive k per thread
-    for (int k0 = 0; k0 < K; k0 += BK) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const int k = k0 + lc + e;
-            xs[lc + e][lr] = (m0 + lr < M && k < K) ? x[(int64_t)(m0 + lr) * ldx + k] : 0.f;
-            ws[lc + e][lr] = (n0 + lr < N && k < K) ? w[(int64_t)(n0 + lr) * ldw + k] : 0.f;
-        }
-        __syncthreads();
-#pragma unroll
-        for (int k = 0; k < BK; ++k) {
-            float a[4], b[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                a[e] = xs[k][tm + e];
-                b[e] = ws[k][tn + e];
-            }
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-#pragma unroll
-                for (int j = 0; j < 4; ++j) acc[i][j] = __builtin_fmaf(a[i], b[j], acc[i][j]);
-        }
-        __syncthreads();
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int m = m0 + tm + i, n = n0 + tn + j;
-            if (m < M && n < N) y[(int64_t)m * ldy + n] = acc[i][j] + (bias ? bias[n] : 0.f);
-        }
+    const int m0 = blockIdx.y * nvh_any::GT;
+    nvh_any::gemm_any_f32_tile(x, ldx, w, ldw, bias, y, ldy, nvh_any::RowMap{nullptr, m0, min(nvh_any::GT, M - m0)}, blockIdx.x * nvh_any::GT, N, K);
 }
 
 }  // namespace
@@ -342,7 +368,7 @@ extern "C" int32_t nvh_gemm_any_nt(const void* x, int64_t x_row_stride, const vo
     NVH_REQUIRE(!in_f32 || out_f32, NVH_ENOSYS, "nvh_gemm_any_nt: fp32 operands give an fp32 product");
     if (M == 0) return NVH_OK;
     hipStream_t st = (hipStream_t)stream;
-    const dim3 grid((unsigned)nvh_cdiv(N, GT), (unsigned)nvh_cdiv(M, GT));
+    const dim3 grid((unsigned)nvh_cdiv(N, nvh_any::GT), (unsigned)nvh_cdiv(M, nvh_any::GT));
     if (in_f32) {
         gemm_any_f32_kernel<<<grid, 256, 0, st>>>((const float*)x, x_row_stride, (const float*)w, K, (const float*)bias, (float*)y, y_row_stride, (int)M, (int)N, (int)K);
     } else {
@@ -351,5 +377,63 @@ extern "C" int32_t nvh_gemm_any_nt(const void* x, int64_t x_row_stride, const vo
         else gemm_any_bf16_kernel<false><<<grid, 256, 0, st>>>((const bf16*)x, x_row_stride, (const bf16*)w, K, (const bf16*)bias, y, y_row_stride, (int)M, (int)N, (int)K, vec_ok);
     }
     NVH_CHECK_LAUNCH("nvh_gemm_any_nt");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_embedding_pos_stream(const int64_t* ids, const int64_t* positions, const void* table, const void* pos_table, float scale,
+                                            float* x, int64_t num_tokens, int64_t dim, int64_t vocab, int64_t max_positions, int32_t act_f32,
+                                            nvh_stream_t stream) {
+    NVH_STREAM_ARGS_OK("nvh_embedding_pos_stream", ids && table && x && num_tokens >= 0 && dim > 0 && vocab > 0 && (!pos_table || (positions && max_positions > 0)));
+    if (num_tokens == 0) return NVH_OK;
+    hipStream_t st = (hipStream_t)stream;
+    if (act_f32) embedding_pos_stream_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(ids, positions, (const float*)table, (const float*)pos_table, scale, x, (int)dim, vocab, max_positions);
+    else embedding_pos_stream_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(ids, positions, (const bf16*)table, (const bf16*)pos_table, scale, x, (int)dim, vocab, max_positions);
+    NVH_CHECK_LAUNCH("nvh_embedding_pos_stream");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_residual_norm(const void* a, int64_t a_stride, const void* a_weight, const void* b, int64_t b_stride, const void* b_weight,
+                                     float branch_scale, float branch_eps, const void* c, int64_t c_stride, const float* c32, int64_t c32_stride,
+                                     float* x, int32_t norm_kind, const void* norm_weight, const void* norm_bias, float eps, void* h, int64_t h_stride,
+                                     int64_t rows, int64_t dim, int32_t act_f32, nvh_stream_t stream) {
+    NVH_STREAM_ARGS_OK("nvh_residual_norm", x && rows >= 0 && dim > 0 && dim <= 32768 && norm_kind >= 0 && norm_kind <= 2 && (norm_kind == 0 || (norm_weight && h)) &&
+                                                (!a_weight || a) && (!b_weight || b));
+    if (rows == 0) return NVH_OK;
+    const CloseArgs p{a, a_weight, b, b_weight, c, c32, a_stride, b_stride, c_stride, c32_stride, branch_scale, branch_eps, x, norm_kind,
+                      norm_weight, norm_bias, eps, h, h_stride, (int)dim};
+    hipStream_t st = (hipStream_t)stream;
+    const size_t lds = sizeof(float) * (size_t)dim;
+    if (lds > 48 * 1024) {
+        const hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(&residual_norm_kernel<float>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        const hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(&residual_norm_kernel<bf16>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        NVH_REQUIRE(e1 == hipSuccess && e2 == hipSuccess, NVH_ENOSYS, "nvh_residual_norm: %zu bytes of LDS refused", lds);
+    }
+    if (act_f32) residual_norm_kernel<float><<<dim3((unsigned)rows), 256, lds, st>>>(p);
+    else residual_norm_kernel<bf16><<<dim3((unsigned)rows), 256, lds, st>>>(p);
+    NVH_CHECK_LAUNCH("nvh_residual_norm");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_act_mul(const void* x, int64_t row_stride, void* y, int64_t y_stride, int64_t rows, int64_t inter, int32_t act, int32_t gated,
+                               int32_t act_f32, nvh_stream_t stream) {
+    NVH_STREAM_ARGS_OK("nvh_act_mul", x && y && rows >= 0 && inter > 0 && act >= 0 && act <= 2 && row_stride >= (gated ? 2 : 1) * inter && y_stride >= inter);
+    if (rows == 0) return NVH_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned blocks = (unsigned)nvh_cdiv(rows * inter, 256);
+    if (act_f32) act_mul_kernel<float><<<dim3(blocks), 256, 0, st>>>((const float*)x, row_stride, (float*)y, y_stride, rows, (int)inter, act, gated);
+    else act_mul_kernel<bf16><<<dim3(blocks), 256, 0, st>>>((const bf16*)x, row_stride, (bf16*)y, y_stride, rows, (int)inter, act, gated);
+    NVH_CHECK_LAUNCH("nvh_act_mul");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_logits_scale(const void* logits, int64_t row_stride, float* out, int64_t rows, int64_t vocab, float scale, float cap,
+                                    int32_t act_f32, nvh_stream_t stream) {
+    NVH_STREAM_ARGS_OK("nvh_logits_scale", logits && out && rows >= 0 && vocab > 0 && row_stride >= vocab);
+    if (rows == 0) return NVH_OK;
+    hipStream_t st = (hipStream_t)stream;
+    const unsigned blocks = (unsigned)nvh_cdiv(rows * vocab, 256);
+    if (act_f32) logits_scale_kernel<float><<<dim3(blocks), 256, 0, st>>>((const float*)logits, row_stride, out, rows, (int)vocab, scale, cap);
+    else logits_scale_kernel<bf16><<<dim3(blocks), 256, 0, st>>>((const bf16*)logits, row_stride, out, rows, (int)vocab, scale, cap);
+    NVH_CHECK_LAUNCH("nvh_logits_scale");
     return NVH_OK;
 }

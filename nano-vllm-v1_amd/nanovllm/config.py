@@ -69,7 +69,8 @@ class Config:
         assert 1 <= self.tensor_parallel_size <= 8
         if self.hf_config is None:
             self.hf_config = load_hf_config(self.model)
-        # (a design whose positions no table bounds has no max_position_embeddings: max_model_len stands as given)
-        self.max_model_len = min(self.max_model_len, getattr(self.hf_config, "max_position_embeddings", None) or self.max_model_len)
+        # (a design whose positions no table bounds names neither max_position_embeddings nor max_positions: max_model_len stands as given)
+        bound = getattr(self.hf_config, "max_position_embeddings", None) or getattr(self.hf_config, "max_positions", None)
+        self.max_model_len = min(self.max_model_len, int(bound) if bound else self.max_model_len)
         if self.num_state_slots <= 0:
             self.num_state_slots = self.max_num_seqs

@@ -105,3 +105,47 @@ class GatedValueRotaryAttention(nn.Module):
                                        self.head_dim, self.value_dim, self.gated, self.interleaved, self.interleaved)
         return ops.attn_paged_any(q, kc, vc, ctx.cu_seqlens_q, ctx.context_lens, ctx.block_tables, self.scale, self.num_heads,
                                   self.num_kv_heads, self.head_dim, self.value_dim, gate, self.value_freq, self.interleaved)
+
+
+class WindowedBiasAttention(nn.Module):
+    """Paged causal attention without rotation whose scores carry a per-head distance bias, score = scale q.k - slope_h (i - j),
+    and whose queries see a sliding window of the last `window` positions plus the first `keep_first` tokens of the sequence
+    (window 0: every earlier token).  Free head sizes (query/key `head_dim`, value `value_dim`), grouped key/value heads.
+
+    Input is the fused projection output [T, H*dim + G*dim + G*vdim] = q | k | v (biases already added).  k and v are
+    scattered to their pages by nvh_attn_rotary_prep (no norm, no rotary), attention runs in nvh_attn_paged_any, which walks
+    only the key tiles a query block can see.  The distance to a kept token is counted from where it really stands, so it
+    grows.  Positions enter nowhere else, so the cache holds keys and values as projected.  One cache pair per pass of a
+    looped stack (`cache_runs`), bound by the runner."""
+
+    def __init__(self, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, scale: float, slopes, window: int = 0,
+                 keep_first: int = 0, cache_runs: int = 1):
+        super().__init__()
+        assert num_heads % num_kv_heads == 0 and window >= 0 and keep_first >= 0
+        self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim = num_heads, num_kv_heads, head_dim, value_dim
+        self.scale, self.window, self.keep_first = scale, window, keep_first
+        slopes = None if slopes is None else torch.as_tensor(slopes, dtype=torch.float64).to(torch.float32)
+        assert slopes is None or slopes.numel() == num_heads
+        self.register_buffer("slopes", None if slopes is None else slopes.to(torch.empty(0).device), persistent=False)
+        self.cache_runs = cache_runs
+        self.k_caches: list = [None] * cache_runs
+        self.v_caches: list = [None] * cache_runs
+
+    @staticmethod
+    def geometric_slopes(num_heads: int, span: float = 8.0) -> list[float]:
+        """slope_h = 2^(-span (h + 1) / H), h = 0 .. H-1: the head-wise geometric sequence of linear distance biases."""
+        return [2.0 ** (-span * (h + 1) / num_heads) for h in range(num_heads)]
+
+    def cache_row_elems(self) -> tuple[int, int]:
+        return self.num_kv_heads * self.head_dim, self.num_kv_heads * self.value_dim
+
+    def forward(self, proj: torch.Tensor, positions: torch.Tensor, run: int = 0) -> torch.Tensor:
+        ctx = get_context()
+        kc, vc = self.k_caches[run], self.v_caches[run]
+        if kc is None or ctx.block_tables is None:
+            raise RuntimeError("this attention reads its keys from the paged cache: bind caches and give every sequence a block table")
+        q, _ = ops.attn_rotary_prep(proj, None, None, 0.0, positions, None, 1.0, 0, None, kc, vc, ctx.slot_mapping, self.num_heads,
+                                    self.num_kv_heads, self.head_dim, self.value_dim, gated=False)
+        return ops.attn_paged_any(q, kc, vc, ctx.cu_seqlens_q, ctx.context_lens, ctx.block_tables, self.scale, self.num_heads,
+                                  self.num_kv_heads, self.head_dim, self.value_dim, slopes=self.slopes, window=self.window,
+                                  keep_first=self.keep_first)

@@ -1,4 +1,6 @@
 """Norm operator modules.  RMSNorm: arithmetic in csrc/elementwise.hip (nvh_rmsnorm / nvh_add_rmsnorm).
+StreamNorm: a layer norm or RMS norm of the fp32 residual stream, applied together with the residual add in front of it by
+nvh_residual_norm (csrc/stream_f32.hip).
 DynamicTanh: a norm without statistics, tanh(alpha x) * weight + bias, applied together with the residual add around
 it by nvh_residual_dyt (csrc/stream_f32.hip) over an fp32 residual stream.
 
@@ -49,3 +51,26 @@ class DynamicTanh(nn.Module):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """x fp32 [rows, dim] -> normalised rows in the parameters' type (x is left as it is)."""
         return ops.residual_dyt(x, nxt=self.triple())
+
+
+class StreamNorm(nn.Module):
+    """Norm of an fp32 residual stream with statistics: kind "layer" = (x - mean) / sqrt(var + eps) * weight + bias (var: the mean
+    squared deviation), kind "rms" = x * rsqrt(mean of squares + eps) * weight.  The module holds the parameters; the arithmetic
+    runs fused with the residual add that precedes it (ops.residual_norm takes `spec()`)."""
+
+    def __init__(self, hidden_size: int, eps: float, kind: str = "layer", bias: bool = True) -> None:
+        super().__init__()
+        assert kind in ("layer", "rms")
+        self.kind, self.eps = kind, eps
+        self.weight = nn.Parameter(torch.ones(hidden_size), requires_grad=False)
+        if bias and kind == "layer":
+            self.bias = nn.Parameter(torch.zeros(hidden_size), requires_grad=False)
+        else:
+            self.register_parameter("bias", None)
+
+    def spec(self) -> dict:
+        return dict(norm=self.kind, weight=self.weight.data, bias=None if self.bias is None else self.bias.data, eps=self.eps)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x fp32 [rows, dim] -> normalised rows in the parameters' type (x is left as it is)."""
+        return ops.residual_norm(x, **self.spec())

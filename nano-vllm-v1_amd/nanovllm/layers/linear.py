@@ -150,9 +150,11 @@ class RowParallelLinear(LinearBase):
 class MergedLinear(nn.Module):
     """Several matrices that read the same input, stored as one weight [sum(out), in] and applied in one product of any
     shape and either activation type (ops.linear_any: the tuned bf16 GEMM where its alignment rules hold, the any-shape
-    kernel otherwise).  Shards are named (`names[i]`); `split(y)` hands back the column views in order.  One rank only."""
+    kernel otherwise).  Shards are named (`names[i]`); `split(y)` hands back the column views in order.  `bias`: a bias per
+    output column, loaded by the same shard names and added inside the product (shards that carry none stay zero).
+    One rank only."""
 
-    def __init__(self, input_size: int, output_sizes: list[int], names: list | None = None):
+    def __init__(self, input_size: int, output_sizes: list[int], names: list | None = None, bias: bool = False):
         super().__init__()
         assert tp_world() == 1, "MergedLinear is not tensor-parallel"
         self.output_sizes = list(output_sizes)
@@ -160,6 +162,11 @@ class MergedLinear(nn.Module):
         self.weight = nn.Parameter(torch.empty(sum(output_sizes), input_size), requires_grad=False)
         self.weight.weight_loader = self.weight_loader
         self.weight.shard_ids = self.shard_ids
+        if bias:
+            self.bias = nn.Parameter(torch.zeros(sum(output_sizes)), requires_grad=False)
+            self.bias.weight_loader = self.weight_loader
+        else:
+            self.register_parameter("bias", None)
 
     def weight_loader(self, param: nn.Parameter, loaded_weight: torch.Tensor, loaded_shard_id=None):
         if loaded_shard_id is None:
@@ -174,4 +181,4 @@ class MergedLinear(nn.Module):
         return y.split(self.output_sizes, dim=-1)
 
     def forward(self, x: torch.Tensor, out_f32: bool = False) -> torch.Tensor:
-        return ops.linear_any(x, self.weight.data, None, out_f32)
+        return ops.linear_any(x, self.weight.data, None if self.bias is None else self.bias.data, out_f32)

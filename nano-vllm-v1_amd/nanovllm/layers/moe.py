@@ -1,0 +1,65 @@
+"""Mixture-of-experts feed-forward: a router picks `top` of `experts` small gated feed-forward layers per token.
+
+    z = W_router h + b            (fp32 logits)
+    picked = the `top` largest z; weights = softmax taken over those `top` values only
+    y = sum_picked weight_e * down_e(act(gate_e h) * up_e h)  (+ shared(h), a gated feed-forward every token passes)
+
+The experts' matrices lie stacked, gate and up merged ([E, 2 ff, D] and [E, D, ff]), and run as two grouped products over
+the (token, choice) pairs ordered by expert (ops.moe_align / ops.linear_grouped); routing, ordering and the tile list stay on
+the device, so a step with experts needs no answer from the host and can be captured in a graph.  The result is the fp32
+sum, meant to be added to an fp32 residual stream.
+"""
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from .. import ops
+from .activation import ActAndMul
+from .linear import MergedLinear
+
+
+class GatedMLP(nn.Module):
+    """down(act(gate x) * up x) with gate and up in one product."""
+
+    def __init__(self, width: int, ff: int, act: str = "silu"):
+        super().__init__()
+        self.gate_up = MergedLinear(width, [ff, ff], ["gate", "up"])
+        self.act = ActAndMul(act)
+        self.down = MergedLinear(ff, [width])
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        return self.down(self.act(self.gate_up(x)))
+
+
+class SparseMoE(nn.Module):
+    def __init__(self, width: int, ff: int, experts: int, top: int, shared_ff: int | None = None, act: str = "silu", router_bias: bool = True):
+        super().__init__()
+        assert 1 <= top <= experts
+        self.width, self.ff, self.experts, self.top, self.act = width, ff, experts, top, act
+        self.router = MergedLinear(width, [experts], bias=router_bias)
+        self.gate_up = nn.Parameter(torch.empty(experts, 2 * ff, width), requires_grad=False)
+        self.down = nn.Parameter(torch.empty(experts, width, ff), requires_grad=False)
+        self.gate_up.weight_loader = self._load_gate_up
+        self.down.weight_loader = self._load_down
+        self.gate_up.shard_ids = [(e, part) for e in range(experts) for part in ("gate", "up")]
+        self.down.shard_ids = list(range(experts))
+        self.shared = GatedMLP(width, shared_ff, act) if shared_ff else None
+
+    def _load_gate_up(self, param: nn.Parameter, loaded_weight: torch.Tensor, shard_id):
+        e, part = shard_id
+        dst = param.data[e].narrow(0, 0 if part == "gate" else self.ff, self.ff)
+        assert dst.shape == loaded_weight.shape, f"expert {e} {part}: {tuple(loaded_weight.shape)} does not fit {tuple(dst.shape)}"
+        dst.copy_(loaded_weight)
+
+    def _load_down(self, param: nn.Parameter, loaded_weight: torch.Tensor, shard_id):
+        assert param.data[shard_id].shape == loaded_weight.shape
+        param.data[shard_id].copy_(loaded_weight)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        """x [T, width] in the activation type -> fp32 [T, width]."""
+        ids, weights = ops.moe_route(self.router(x, out_f32=True), self.top)
+        plan = ops.moe_align(ids, self.experts)
+        hidden = ops.act_mul(ops.linear_grouped(x, self.gate_up.data, plan, gather=True), self.act, True)
+        y = ops.linear_grouped(hidden, self.down.data, plan, gather=False)
+        return ops.moe_combine(y, plan, weights, self.shared(x) if self.shared is not None else None)

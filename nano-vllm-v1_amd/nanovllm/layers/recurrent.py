@@ -13,6 +13,7 @@ from torch import nn
 
 from .. import ops
 from ..utils.context import get_context
+from .linear import MergedLinear
 
 
 class GeneralizedDeltaRule(nn.Module):
@@ -50,3 +51,120 @@ class GeneralizedDeltaRule(nn.Module):
         o = ops.delta_rule(r, k, v, a_raw, lowrank, self.w2.data, self.w0.data, self.a_bias.data, state, ctx.state_slots,
                            ctx.cu_seqlens_q, ctx.context_lens, self.num_heads, self.head_dim, self.decay_scale)
         return ops.delta_post(o, self.norm.data, g, self.num_heads, self.head_dim, self.eps)
+
+
+class _StatePool(nn.Module):
+    """A per-sequence fp32 state of fixed shape, one pool [slots, *shape] per pass (`states[run]`, bound by the runner)."""
+
+    def __init__(self, shape: tuple, state_runs: int = 1):
+        super().__init__()
+        self._shape = tuple(int(n) for n in shape)
+        self.state_runs = state_runs
+        self.states: list = [None] * state_runs
+
+    def state_shape(self) -> tuple:
+        return self._shape
+
+    def pool(self, run: int) -> torch.Tensor:
+        ctx = get_context()
+        if self.states[run] is None or ctx.state_slots is None:
+            raise RuntimeError("a recurrent layer needs a bound state pool and a state slot per sequence")
+        return self.states[run]
+
+
+class DiagonalDecayRecurrence(_StatePool):
+    """Per head a matrix memory S [dk, dv] in fp32 with a diagonal decay:
+
+        S <- diag(w) S + (c k) v^T,      o = S^T q + d v
+
+    w: one decay for each key channel, or a single one per head, c: a write strength per head (None: 1), d: a skip weight per head (None: 0),
+    q and k possibly shared by groups of heads.  The operands are fp32 (the mixers below make them from their projections);
+    the scan walks this step's tokens of every sequence from the state its slot holds, or from zero when the sequence
+    starts in this step (kernel: nvh_gated_linear_scan, csrc/linear_recurrence.hip)."""
+
+    def __init__(self, num_heads: int, key_dim: int, value_dim: int, qk_groups: int | None = None, state_runs: int = 1):
+        super().__init__((num_heads, key_dim, value_dim), state_runs)
+        self.num_heads, self.key_dim, self.value_dim, self.qk_groups = num_heads, key_dim, value_dim, qk_groups or num_heads
+
+    def forward(self, q, k, w, v, run: int = 0, kscale=None, skip=None) -> torch.Tensor:
+        state = self.pool(run)
+        ctx = get_context()
+        return ops.gated_linear_scan(q, k, w, v, state, ctx.state_slots, ctx.cu_seqlens_q, ctx.context_lens, self.num_heads, self.key_dim,
+                                     self.value_dim, self.qk_groups, kscale, skip)
+
+
+class HGRN2(nn.Module):
+    """HGRN2 cell: a linear-attention memory without a key, the forget gate's complement taking its place.  Per head and key channel
+    g = lower + (1 - lower) sigmoid(f + f_bias) in [lower, 1); S <- diag(g) S + (1 - g) v^T; o = S^T silu(q); q is the only
+    other operand.  The read-out of a head is normalised (RMS along value_dim) by a single weight vector common to the heads.
+
+    forward takes the column views q, f, v of the fused projection and returns [T, H * value_dim] in the activation type."""
+
+    def __init__(self, num_heads: int, key_dim: int, value_dim: int, eps: float, state_runs: int = 1):
+        super().__init__()
+        n = num_heads * key_dim
+        self.num_heads, self.key_dim, self.value_dim, self.eps = num_heads, key_dim, value_dim, eps
+        self.f_bias = nn.Parameter(torch.zeros(n), requires_grad=False)
+        self.lower = nn.Parameter(torch.zeros(n), requires_grad=False)
+        self.norm = nn.Parameter(torch.ones(value_dim), requires_grad=False)
+        self.memory = DiagonalDecayRecurrence(num_heads, key_dim, value_dim, state_runs=state_runs)
+
+    def forward(self, q, f, v, run: int = 0) -> torch.Tensor:
+        o = self.memory(*ops.hgrn2_prep(q, f, v, self.f_bias.data, self.lower.data), run)
+        return ops.group_rmsnorm_gate(o, self.norm.data, self.value_dim, self.eps)
+
+
+class GatedLinearAttention(nn.Module):
+    """Gated linear attention: S <- diag(alpha) S + k v^T, o = S^T (q / sqrt(key_dim)), where every key channel has its own decay
+    alpha = exp(log_sigmoid(z) / tau), z = W2 (low-rank input) + bias.  The read-out of a head is normalised (RMS along value_dim, a
+    single weight vector common to the heads) and then gated by silu(gate).
+
+    forward takes the column views q, k, v, gate and the low-rank decay input of the fused projection."""
+
+    def __init__(self, num_heads: int, key_dim: int, value_dim: int, rank: int, tau: float, eps: float, state_runs: int = 1):
+        super().__init__()
+        self.num_heads, self.key_dim, self.value_dim, self.tau, self.eps = num_heads, key_dim, value_dim, float(tau), eps
+        self.decay_up = MergedLinear(rank, [num_heads * key_dim], bias=True)          # W2 and its bias
+        self.norm = nn.Parameter(torch.ones(value_dim), requires_grad=False)
+        self.memory = DiagonalDecayRecurrence(num_heads, key_dim, value_dim, state_runs=state_runs)
+
+    def forward(self, q, k, v, gate, lowrank, run: int = 0) -> torch.Tensor:
+        z = self.decay_up(lowrank, out_f32=True)
+        o = self.memory(*ops.gla_prep(q, k, v, z, self.key_dim ** -0.5, self.tau), run)
+        return ops.group_rmsnorm_gate(o, self.norm.data, self.value_dim, self.eps, gate, "silu", gate_first=False)
+
+
+class Mamba2(nn.Module):
+    """The state-space-duality layer of Mamba-2.  The in-projection row holds z and x (inner = H * value_dim wide each), then B and C
+    (groups * state_dim each), then one dt per head.  x, B, C pass a causal depthwise convolution (`taps` wide, last tap on the current token, continued
+    across steps from the sequence's last taps - 1 inputs) and silu; dt = softplus(dt + dt_bias), unclamped.  Per head (B, C
+    shared by the heads of a group):  S <- exp(-exp(A_log) dt) S + dt B x^T,  y = S^T C + D x,  S [N, value_dim] fp32.
+    Read-out: y * silu(z), then an RMS norm taken separately over `norm_groups` equal slices, with a weight per column (gated, then normalised).
+
+    forward takes the whole projection row and returns [T, inner] in the activation type."""
+
+    def __init__(self, num_heads: int, value_dim: int, state_dim: int, groups: int, taps: int, norm_groups: int, eps: float, state_runs: int = 1):
+        super().__init__()
+        assert num_heads % groups == 0 and (num_heads * value_dim) % norm_groups == 0
+        self.num_heads, self.value_dim, self.state_dim, self.groups, self.taps, self.norm_groups, self.eps = num_heads, value_dim, state_dim, groups, taps, norm_groups, eps
+        self.inner, self.gn = num_heads * value_dim, groups * state_dim
+        channels = self.inner + 2 * self.gn
+        self.conv_weight = nn.Parameter(torch.zeros(channels, taps), requires_grad=False)
+        self.conv_bias = nn.Parameter(torch.zeros(channels), requires_grad=False)
+        self.dt_bias = nn.Parameter(torch.zeros(num_heads), requires_grad=False)
+        self.A_log = nn.Parameter(torch.zeros(num_heads), requires_grad=False)
+        self.D = nn.Parameter(torch.ones(num_heads, dtype=torch.float32), requires_grad=False)      # (an operand of the fp32 scan)
+        self.norm = nn.Parameter(torch.ones(self.inner), requires_grad=False)
+        self.conv_inputs = _StatePool((max(taps - 1, 1), channels), state_runs)     # the last taps - 1 inputs of x | B | C per sequence
+        self.memory = DiagonalDecayRecurrence(num_heads, state_dim, value_dim, qk_groups=groups, state_runs=state_runs)
+
+    def projection_sizes(self) -> list[int]:
+        return [self.inner, self.inner + 2 * self.gn, self.num_heads]               # z | x B C | dt
+
+    def forward(self, z, xbc, dt, run: int = 0) -> torch.Tensor:
+        ctx = get_context()
+        x, b, c, step, decay = ops.ssd_conv_prep(xbc, dt, self.conv_weight.data, self.conv_bias.data, self.dt_bias.data, self.A_log.data,
+                                                 self.conv_inputs.pool(run), ctx.state_slots, ctx.cu_seqlens_q, ctx.context_lens,
+                                                 self.num_heads, self.inner, self.gn)
+        y = self.memory(c, b, decay, x, run, kscale=step, skip=self.D.data)
+        return ops.group_rmsnorm_gate(y, self.norm.data, self.inner // self.norm_groups, self.eps, z, "silu", gate_first=True)

@@ -18,6 +18,8 @@ _REGISTRY = {
     "Qwen2ForCausalLM": ("qwen3", "Qwen3ForCausalLM"),        # the same wiring with attention_bias (models/qwen3.py)
     "Lamutar": ("lamutar", "LamutarForCausalLM"),
     "LamutarForCausalLM": ("lamutar", "LamutarForCausalLM"),
+    "Dinatar": ("dinatar", "DinatarForCausalLM"),
+    "DinatarForCausalLM": ("dinatar", "DinatarForCausalLM"),
 }
 
 

@@ -660,25 +660,27 @@ def attn_rotary_prep(proj, q_norm, k_norm, eps: float, positions, qk_freq, qk_ma
                      slot_mapping, heads: int, kv_heads: int, dim: int, vdim: int, gated: bool = True, qk_interleaved: bool = False,
                      v_interleaved: bool = False):
     """(q [T, H*dim], sigmoid gate fp32 [T, H] | None) from the fused projection rows [q | k | v | gate]; k and v go to their
-    cache rows (see nvh_attn_rotary_prep)."""
-    f = _act_flag(proj, q_norm, k_norm, k_cache, v_cache)
+    cache rows (see nvh_attn_rotary_prep).  q_norm / k_norm None: no norm; rot_dims 0: no rotary."""
+    f = _act_flag(proj, k_cache, v_cache) if q_norm is None else _act_flag(proj, q_norm, k_norm, k_cache, v_cache)
     t = proj.shape[0]
     assert proj.stride(1) == 1 and positions.dtype == torch.int64 and slot_mapping.dtype == torch.int32 and slot_mapping.numel() == t
     assert qk_freq is None or (qk_freq.dtype == F32 and qk_freq.numel() * 2 == rot_dims)
     assert v_freq is None or (v_freq.dtype == F32 and v_freq.numel() * 2 == vdim)
-    assert q_norm.numel() == heads * dim and k_norm.numel() == kv_heads * dim and k_cache.is_contiguous() and v_cache.is_contiguous()
+    assert (q_norm is None and k_norm is None) or (q_norm.numel() == heads * dim and k_norm.numel() == kv_heads * dim)
+    assert k_cache.is_contiguous() and v_cache.is_contiguous()
     q = torch.empty(t, heads * dim, dtype=proj.dtype, device=proj.device)
     gate = torch.empty(t, heads, dtype=F32, device=proj.device) if gated else None
-    _hip.call("nvh_attn_rotary_prep", proj.data_ptr(), proj.stride(0), q_norm.data_ptr(), k_norm.data_ptr(), float(eps), positions.data_ptr(),
+    _hip.call("nvh_attn_rotary_prep", proj.data_ptr(), proj.stride(0), _p(q_norm), _p(k_norm), float(eps), positions.data_ptr(),
               _p(qk_freq), float(qk_mag), rot_dims, int(qk_interleaved), _p(v_freq), int(v_interleaved), q.data_ptr(), _p(gate),
               k_cache.data_ptr(), v_cache.data_ptr(), slot_mapping.data_ptr(), k_cache.shape[1], t, heads, kv_heads, dim, vdim, f, _stream())
     return q, gate
 
 
 def attn_paged_any(q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables, scale: float, heads: int, kv_heads: int, dim: int,
-                   vdim: int, gate=None, v_freq=None, v_interleaved: bool = False) -> torch.Tensor:
+                   vdim: int, gate=None, v_freq=None, v_interleaved: bool = False, slopes=None, window: int = 0, keep_first: int = 0) -> torch.Tensor:
     """Causal attention of the packed queries q [T, H*dim] over paged caches, keys [pages, page, G, dim] and values
-    [pages, G, vdim, page] (transposed within a page, as attn_rotary_prep stores them); out [T, H*vdim]."""
+    [pages, G, vdim, page] (transposed within a page, as attn_rotary_prep stores them); out [T, H*vdim].  `slopes` (fp32 [H]):
+    score -= slope * distance; `window` > 0: a query sees the last `window` positions and the first `keep_first`."""
     f = _act_flag(q, k_cache, v_cache)
     t = q.shape[0]
     batch = context_lens.numel()
@@ -688,10 +690,11 @@ def attn_paged_any(q, k_cache, v_cache, cu_seqlens_q, context_lens, block_tables
     assert cu_seqlens_q is None or (cu_seqlens_q.dtype == torch.int32 and cu_seqlens_q.numel() == batch + 1)
     assert cu_seqlens_q is not None or t == batch
     assert gate is None or (gate.dtype == F32 and gate.shape == (t, heads) and gate.is_contiguous())
+    assert slopes is None or (slopes.dtype == F32 and slopes.numel() == heads and slopes.is_contiguous() and slopes.is_cuda)
     out = torch.empty(t, heads * vdim, dtype=q.dtype, device=q.device)
     _hip.call("nvh_attn_paged_any", q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(),
               block_tables.data_ptr(), block_tables.stride(0), batch, t, k_cache.shape[1], heads, kv_heads, dim, vdim, float(scale),
-              _p(gate), _p(v_freq), int(v_interleaved), out.data_ptr(), f, _stream())
+              _p(gate), _p(v_freq), int(v_interleaved), _p(slopes), int(window), int(keep_first), out.data_ptr(), f, _stream())
     return out
 
 
@@ -726,3 +729,201 @@ def delta_post(o: torch.Tensor, norm_weight: torch.Tensor, gate: torch.Tensor | 
     _hip.call("nvh_delta_post", o.data_ptr(), norm_weight.data_ptr(), _p(gate), gate.stride(0) if gate is not None else 0, y.data_ptr(),
               y.stride(0), o.shape[0], heads, dv, float(eps), f, _stream())
     return y
+
+
+# ---------------------------------------------------------------- layer norm / RMS norm around the fp32 stream, plain activations
+NORM_KINDS = {None: 0, "layer": 1, "rms": 2}
+ACTS = {"silu": 0, "gelu_tanh": 1, "relu2": 2}
+
+
+def embedding_pos_stream(ids: torch.Tensor, positions: torch.Tensor, table: torch.Tensor, pos_table: torch.Tensor | None, scale: float = 1.0) -> torch.Tensor:
+    """fp32 rows table[ids] * scale + pos_table[positions]."""
+    f = _act_flag(table) if pos_table is None else _act_flag(table, pos_table)
+    assert ids.dtype == torch.int64 and positions.dtype == torch.int64 and table.is_contiguous() and (pos_table is None or pos_table.is_contiguous())
+    t, dim = ids.numel(), table.shape[1]
+    assert pos_table is None or pos_table.shape[1] == dim
+    x = torch.empty(t, dim, dtype=F32, device=table.device)
+    _hip.call("nvh_embedding_pos_stream", ids.data_ptr(), positions.data_ptr(), table.data_ptr(), _p(pos_table), float(scale), x.data_ptr(), t, dim,
+              table.shape[0], pos_table.shape[0] if pos_table is not None else 0, f, _stream())
+    return x
+
+
+def residual_norm(x: torch.Tensor, a=None, a_weight=None, b=None, b_weight=None, branch_scale: float = 1.0, branch_eps: float = 0.0, c=None, c32=None,
+                  norm: str | None = None, weight=None, bias=None, eps: float = 0.0) -> torch.Tensor | None:
+    """x <- x + branch_scale * (unit(a) a_weight + unit(b) b_weight) + c + c32 in place (fp32 rows; a branch without a weight
+    is added as it is, absent terms are skipped); returns norm(x) in the activation type, or None without `norm`."""
+    assert x.dtype == F32 and x.is_contiguous() and x.dim() == 2
+    rows, dim = x.shape
+    typed = [t for t in (a, a_weight, b, b_weight, c, weight, bias) if t is not None]
+    assert typed, "nothing to add and nothing to normalise"
+    f = _act_flag(*typed)
+    for t in (a, b, c):
+        assert t is None or (t.shape == (rows, dim) and t.stride(1) == 1)
+    for t in (a_weight, b_weight, weight, bias):
+        assert t is None or (t.numel() == dim and t.is_contiguous())
+    assert c32 is None or (c32.dtype == F32 and c32.shape == (rows, dim) and c32.stride(1) == 1)
+    h = torch.empty(rows, dim, dtype=weight.dtype, device=x.device) if norm is not None else None
+    _hip.call("nvh_residual_norm", _p(a), a.stride(0) if a is not None else 0, _p(a_weight), _p(b), b.stride(0) if b is not None else 0, _p(b_weight),
+              float(branch_scale), float(branch_eps), _p(c), c.stride(0) if c is not None else 0, _p(c32), c32.stride(0) if c32 is not None else 0,
+              x.data_ptr(), NORM_KINDS[norm], _p(weight), _p(bias), float(eps), _p(h), dim, rows, dim, f, _stream())
+    return h
+
+
+def act_mul(x: torch.Tensor, act: str, gated: bool) -> torch.Tensor:
+    """act(x) for plain rows, act(x[:, :I]) * x[:, I:] for a merged [gate | up] projection; act: silu, gelu_tanh, relu2."""
+    f = _act_flag(x)
+    assert x.dim() == 2 and x.stride(1) == 1
+    rows, inter = x.shape[0], x.shape[1] // 2 if gated else x.shape[1]
+    y = torch.empty(rows, inter, dtype=x.dtype, device=x.device)
+    _hip.call("nvh_act_mul", x.data_ptr(), x.stride(0), y.data_ptr(), inter, rows, inter, ACTS[act], int(gated), f, _stream())
+    return y
+
+
+def logits_scale(logits: torch.Tensor, scale: float, cap: float = 0.0) -> torch.Tensor:
+    """fp32 scale * logits (softcapped when cap > 0)."""
+    f = _act_flag(logits)
+    assert logits.dim() == 2 and logits.stride(1) == 1
+    out = torch.empty(logits.shape, dtype=F32, device=logits.device)
+    _hip.call("nvh_logits_scale", logits.data_ptr(), logits.stride(0), out.data_ptr(), logits.shape[0], logits.shape[1], float(scale), float(cap or 0.0), f, _stream())
+    return out
+
+
+# ---------------------------------------------------------------- linear recurrences with a diagonal decay
+def _f32_rows(t, *tensors):
+    for x in tensors:
+        assert x.dtype == F32 and x.is_cuda and x.stride(-1) == 1 and x.shape[0] == t
+
+
+def gated_linear_scan(q, k, w, v, state, slots, cu_seqlens_q, context_lens, heads: int, dk: int, dv: int, qk_groups: int | None = None,
+                      kscale=None, skip=None) -> torch.Tensor:
+    """S <- diag(w) S + (kscale k) v^T, o = S^T q + skip v over the packed tokens; fp32 operands q, k [T, qk_groups * dk],
+    w [T, H * dk] or [T, H] (one decay per head), kscale [T, H] | None, v [T, H * dv], skip [H] | None; `state`
+    [slots, H, dk, dv] fp32 is read (unless the sequence starts in this step) and left updated.  Returns fp32 [T, H * dv]."""
+    t = v.shape[0]
+    g = qk_groups or heads
+    _f32_rows(t, q, k, w, v)
+    assert q.shape[1] == g * dk and k.shape[1] == g * dk and v.shape[1] == heads * dv and w.shape[1] in (heads, heads * dk)
+    w_scalar = w.shape[1] == heads and dk != 1
+    assert kscale is None or (kscale.dtype == F32 and kscale.shape == (t, heads) and kscale.stride(1) == 1)
+    assert skip is None or (skip.dtype == F32 and skip.numel() == heads and skip.is_contiguous())
+    assert state.dtype == F32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dk, dv) and slots.dtype == torch.int32
+    assert context_lens.dtype == torch.int32 and (cu_seqlens_q is None or cu_seqlens_q.dtype == torch.int32)
+    batch = context_lens.numel()
+    assert cu_seqlens_q is not None or t == batch
+    out = torch.empty(t, heads * dv, dtype=F32, device=v.device)
+    _hip.call("nvh_gated_linear_scan", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), g, w.data_ptr(), w.stride(0), int(w_scalar),
+              _p(kscale), kscale.stride(0) if kscale is not None else 0, v.data_ptr(), v.stride(0), _p(skip), state.data_ptr(), slots.data_ptr(),
+              _p(cu_seqlens_q), context_lens.data_ptr(), out.data_ptr(), batch, heads, dk, dv, _stream())
+    return out
+
+
+def hgrn2_prep(q, f, v, f_bias, lower):
+    """fp32 (q, k, w, v) of the HGRN2 recurrence from projection columns: silu(q), 1 - g, g = lower + (1 - lower) sigmoid(f + f_bias), v."""
+    fl = _act_flag(q, f, v, f_bias, lower)
+    t, nk, nv = q.shape[0], q.shape[1], v.shape[1]
+    assert q.stride(1) == 1 and f.stride(1) == 1 and v.stride(1) == 1 and f.shape == (t, nk) and f_bias.numel() == nk and lower.numel() == nk
+    oq, ok, ow = (torch.empty(t, nk, dtype=F32, device=q.device) for _ in range(3))
+    ov = torch.empty(t, nv, dtype=F32, device=q.device)
+    _hip.call("nvh_hgrn2_prep", q.data_ptr(), q.stride(0), f.data_ptr(), f.stride(0), v.data_ptr(), v.stride(0), f_bias.data_ptr(), lower.data_ptr(),
+              oq.data_ptr(), ok.data_ptr(), ow.data_ptr(), ov.data_ptr(), t, nk, nv, fl, _stream())
+    return oq, ok, ow, ov
+
+
+def gla_prep(q, k, v, decay_logits, q_scale: float, tau: float):
+    """fp32 (q * q_scale, k, sigmoid(decay_logits)^(1/tau), v) from projection columns and fp32 decay logits."""
+    fl = _act_flag(q, k, v)
+    t, nk, nv = q.shape[0], q.shape[1], v.shape[1]
+    assert q.stride(1) == 1 and k.stride(1) == 1 and v.stride(1) == 1 and k.shape == (t, nk)
+    assert decay_logits.dtype == F32 and decay_logits.shape == (t, nk) and decay_logits.stride(1) == 1
+    oq, ok, ow = (torch.empty(t, nk, dtype=F32, device=q.device) for _ in range(3))
+    ov = torch.empty(t, nv, dtype=F32, device=q.device)
+    _hip.call("nvh_gla_prep", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), v.data_ptr(), v.stride(0), decay_logits.data_ptr(),
+              decay_logits.stride(0), float(q_scale), float(tau), oq.data_ptr(), ok.data_ptr(), ow.data_ptr(), ov.data_ptr(), t, nk, nv, fl, _stream())
+    return oq, ok, ow, ov
+
+
+def ssd_conv_prep(xbc, dt, conv_w, conv_b, dt_bias, a_log, conv_state, slots, cu_seqlens_q, context_lens, heads: int, inner: int, gn: int):
+    """Causal convolution + silu over the channels x | B | C of the in-projection (continued from `conv_state`
+    [slots, taps - 1, C] fp32, which is then brought up to date), dt = softplus(dt + dt_bias), decay = exp(-exp(a_log) dt):
+    fp32 (x [T, inner], B [T, gn], C [T, gn], dt [T, H], decay [T, H])."""
+    fl = _act_flag(xbc, dt, conv_w, dt_bias, a_log)
+    t, c = xbc.shape[0], inner + 2 * gn
+    taps = conv_w.shape[1]
+    assert xbc.shape[1] == c and xbc.stride(1) == 1 and dt.shape == (t, heads) and dt.stride(1) == 1 and conv_w.shape == (c, taps) and conv_w.is_contiguous()
+    assert conv_b is None or (conv_b.numel() == c and conv_b.dtype == conv_w.dtype)
+    assert taps == 1 or (conv_state.dtype == F32 and conv_state.is_contiguous() and tuple(conv_state.shape[1:]) == (taps - 1, c))
+    assert slots.dtype == torch.int32 and context_lens.dtype == torch.int32 and (cu_seqlens_q is None or cu_seqlens_q.dtype == torch.int32)
+    batch = context_lens.numel()
+    ox = torch.empty(t, inner, dtype=F32, device=xbc.device)
+    ob, oc = (torch.empty(t, gn, dtype=F32, device=xbc.device) for _ in range(2))
+    odt, odecay = (torch.empty(t, heads, dtype=F32, device=xbc.device) for _ in range(2))
+    _hip.call("nvh_ssd_conv_prep", xbc.data_ptr(), xbc.stride(0), dt.data_ptr(), dt.stride(0), conv_w.data_ptr(), _p(conv_b), dt_bias.data_ptr(),
+              a_log.data_ptr(), _p(conv_state), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(), batch, t, taps, heads, inner, gn,
+              ox.data_ptr(), ob.data_ptr(), oc.data_ptr(), odt.data_ptr(), odecay.data_ptr(), fl, _stream())
+    _hip.call("nvh_conv_state_update", xbc.data_ptr(), xbc.stride(0), _p(conv_state), slots.data_ptr(), _p(cu_seqlens_q), context_lens.data_ptr(), batch,
+              taps, c, fl, _stream())
+    return ox, ob, oc, odt, odecay
+
+
+def group_rmsnorm_gate(o: torch.Tensor, weight: torch.Tensor, group_size: int, eps: float, gate=None, gate_act: str | None = None,
+                       gate_first: bool = False) -> torch.Tensor:
+    """RMS norm of fp32 rows over groups of `group_size` columns, times `weight` ([group_size], shared by the groups, or one per
+    column), with an optional gate (columns of the activation type; "sigmoid" or "silu") applied before or after the norm."""
+    f = _act_flag(weight) if gate is None else _act_flag(weight, gate)
+    rows, n = o.shape
+    assert o.dtype == F32 and o.is_contiguous() and n % group_size == 0 and weight.numel() in (group_size, n) and weight.is_contiguous()
+    assert gate is None or (gate.shape == (rows, n) and gate.stride(1) == 1 and gate_act in ("sigmoid", "silu"))
+    y = torch.empty(rows, n, dtype=weight.dtype, device=o.device)
+    _hip.call("nvh_group_rmsnorm_gate", o.data_ptr(), weight.data_ptr(), int(weight.numel() == n and n != group_size), _p(gate),
+              gate.stride(0) if gate is not None else 0, {None: 0, "sigmoid": 1, "silu": 2}[gate_act if gate is not None else None], int(gate_first),
+              y.data_ptr(), n, rows, n // group_size, group_size, float(eps), f, _stream())
+    return y
+
+
+# ---------------------------------------------------------------- mixture of experts
+def moe_route(logits: torch.Tensor, top: int):
+    """(ids int32 [T, top], weights fp32 [T, top]): the `top` largest fp32 router logits per token, softmax over them alone."""
+    assert logits.dtype == F32 and logits.dim() == 2 and logits.stride(1) == 1 and logits.is_cuda
+    t, e = logits.shape
+    ids = torch.empty(t, top, dtype=torch.int32, device=logits.device)
+    weights = torch.empty(t, top, dtype=F32, device=logits.device)
+    _hip.call("nvh_moe_route", logits.data_ptr(), logits.stride(0), ids.data_ptr(), weights.data_ptr(), t, e, top, _stream())
+    return ids, weights
+
+
+def moe_align(ids: torch.Tensor, experts: int) -> dict:
+    """The (token, choice) pairs ordered by expert, as device arrays (see nvh_moe_align): src_token, pos_of_pair, and the tile list."""
+    assert ids.dtype == torch.int32 and ids.is_contiguous() and ids.is_cuda
+    t, top = ids.shape
+    pairs = t * top
+    max_tiles = int(_hip.lib().nvh_moe_max_tiles(pairs, experts))
+    buf = torch.empty(2 * pairs + 3 * max_tiles, dtype=torch.int32, device=ids.device)
+    src, pos = buf[:pairs], buf[pairs:2 * pairs]
+    te, t0, tr = (buf[2 * pairs + i * max_tiles:2 * pairs + (i + 1) * max_tiles] for i in range(3))
+    _hip.call("nvh_moe_align", ids.data_ptr(), t, experts, top, src.data_ptr(), pos.data_ptr(), te.data_ptr(), t0.data_ptr(), tr.data_ptr(), max_tiles, _stream())
+    return dict(src_token=src, pos_of_pair=pos, tile_expert=te, tile_row0=t0, tile_rows=tr, max_tiles=max_tiles, pairs=pairs)
+
+
+def linear_grouped(x: torch.Tensor, weight: torch.Tensor, plan: dict, gather: bool, out_f32: bool = False) -> torch.Tensor:
+    """y[pos] = x[src_token[pos] if gather else pos] @ weight[expert of pos]^T for every position of the plan; weight [E, N, K]."""
+    f = _act_flag(x, weight)
+    e, n, k = weight.shape
+    assert weight.is_contiguous() and x.dim() == 2 and x.shape[1] == k and x.stride(1) == 1 and (gather or x.shape[0] == plan["pairs"])
+    out_f32 = bool(out_f32 or f)
+    y = torch.empty(plan["pairs"], n, dtype=F32 if out_f32 else BF16, device=x.device)
+    _hip.call("nvh_gemm_grouped_any_nt", x.data_ptr(), x.stride(0), plan["src_token"].data_ptr() if gather else 0, weight.data_ptr(), y.data_ptr(), n,
+              plan["tile_expert"].data_ptr(), plan["tile_row0"].data_ptr(), plan["tile_rows"].data_ptr(), plan["max_tiles"], n, k, f, int(out_f32), _stream())
+    return y
+
+
+def moe_combine(y: torch.Tensor, plan: dict, weights: torch.Tensor, shared: torch.Tensor | None = None) -> torch.Tensor:
+    """fp32 [T, dim]: every token's weighted sum of its choices' rows of y (in choice order), plus `shared` [T, dim]."""
+    f = _act_flag(y) if shared is None else _act_flag(y, shared)
+    t, top = weights.shape
+    dim = y.shape[1]
+    assert y.stride(1) == 1 and weights.dtype == F32 and weights.is_contiguous() and y.shape[0] == t * top
+    assert shared is None or (shared.shape == (t, dim) and shared.stride(1) == 1)
+    out = torch.empty(t, dim, dtype=F32, device=y.device)
+    _hip.call("nvh_moe_combine", y.data_ptr(), y.stride(0), plan["pos_of_pair"].data_ptr(), weights.data_ptr(), _p(shared),
+              shared.stride(0) if shared is not None else 0, out.data_ptr(), t, dim, top, f, _stream())
+    return out
