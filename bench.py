@@ -464,35 +464,60 @@ HYBRID_SIZES = {
 }
 
 
+def _lamutar_cfg(z):
+    attn = {"type": "attention", "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["head_dim"], "vdim": z["head_dim"],
+                                           "scale": z["head_dim"] ** -0.5,
+                                           "rot": {"base": 1e6, "dims": z["head_dim"] // 2, "scaling": {"factor": 4.0, "original": 4096, "fast": 16.0, "slow": 2.0}}},
+            "mlp": {"kind": "dense", "ff": z["ff"]}}
+    delta = {"type": "general_delta", "mixer": {"heads": z["width"] // 64, "dim": 64}, "mlp": {"kind": "dense", "ff": z["ff"]}}
+    return {"architecture": "Lamutar", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "loop": None,
+            "layers": [attn if i % 2 == 1 else delta for i in range(z["layers"])]}
+
+
+def _qwen3_cfg(z):
+    return {"architectures": ["Qwen3ForCausalLM"], "hidden_size": z["width"], "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
+            "num_key_value_heads": z["kv_heads"], "head_dim": z["head_dim"], "intermediate_size": z["ff"], "vocab_size": z["vocab"],
+            "max_position_embeddings": 40960, "rms_norm_eps": 1e-6, "rope_theta": 1000000, "tie_word_embeddings": False, "hidden_act": "silu",
+            "attention_bias": False, "torch_dtype": "bfloat16"}
+
+
+def _dinatar_cfg(z):
+    """Parallel (windowed attention beside Mamba-2), HGRN2 and gated-linear-attention layers in turn; dense and mixture-of-experts
+    feed-forwards in turn, the experts sized so that a token passes about as many feed-forward weights as in the dense layers."""
+    w, hd = z["width"], z["head_dim"]
+    par = {"left": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": hd, "vdim": hd, "scale": hd ** -0.5, "mask": {"size": 512, "keep_first": 4}},
+           "right": {"heads": 2 * w // 64, "vdim": 64, "state": 128, "groups": 8, "conv": 4, "norm_groups": 1}}
+    mixers = [("parallel", par), ("hgrn2", {"heads": w // 128, "dim": 128, "vdim": 128}), ("gla", {"heads": w // 256, "dim": 128, "vdim": 256, "tau": 16.0})]
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "expert": {"ff": z["ff"] // 8}, "router": {"experts": 16, "top": 2}, "shared": {"ff": z["ff"] // 4}}
+    return {"architecture": "Dinatar", "vocab": z["vocab"], "width": w, "max_positions": 8192, "embedding": {"scale": 1.0}, "logit_scale": 1.0,
+            "norm": {"eps": 1e-5}, "loop": None,
+            "layers": [{"type": mixers[i % 3][0], "mixer": mixers[i % 3][1], "mlp": moe if i % 2 else dense} for i in range(z["layers"])]}
+
+
+HYBRID_DESIGNS = {
+    # --hybrid-design: (the design, the closest model the engine already serves)
+    "lamutar": (("lamutar", _lamutar_cfg), ("qwen3", _qwen3_cfg)),
+    "dinatar": (("dinatar", _dinatar_cfg), ("lamutar", _lamutar_cfg)),
+}
+
+
 def hybrid_compare(args):
-    """--hybrid-compare: prefill and decode throughput of the Lamutar design (delta-rule and attention layers in turn, fp32 residual
-    stream, operator modules + captured decode graphs) beside Qwen3 (the closest model the engine serves: native executor)
-    at equal width, heads, feed-forward size, depth and vocabulary; random weights, bf16.  One JSON line."""
+    """--hybrid-compare: prefill and decode throughput of a hybrid design (--hybrid-design; operator modules over an fp32 residual
+    stream + captured decode graphs) beside the closest model the engine serves at equal width, heads, feed-forward size, depth and
+    vocabulary: Lamutar (delta-rule and attention layers in turn) beside Qwen3 (native executor), or Dinatar (windowed attention +
+    Mamba-2, HGRN2, gated linear attention; dense and expert feed-forwards) beside Lamutar.  Random weights, bf16.  One JSON line."""
     import tempfile
     from nanovllm.config import Config
     from nanovllm.engine.model_runner import ModelRunner
 
-    def lamutar_cfg(z):
-        attn = {"type": "attention", "mixer": {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["head_dim"], "vdim": z["head_dim"],
-                                               "scale": z["head_dim"] ** -0.5,
-                                               "rot": {"base": 1e6, "dims": z["head_dim"] // 2, "scaling": {"factor": 4.0, "original": 4096, "fast": 16.0, "slow": 2.0}}},
-                "mlp": {"kind": "dense", "ff": z["ff"]}}
-        delta = {"type": "general_delta", "mixer": {"heads": z["width"] // 64, "dim": 64}, "mlp": {"kind": "dense", "ff": z["ff"]}}
-        return {"architecture": "Lamutar", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "logit_softcap": 30.0, "loop": None,
-                "layers": [attn if i % 2 == 1 else delta for i in range(z["layers"])]}
-
-    def qwen3_cfg(z):
-        return {"architectures": ["Qwen3ForCausalLM"], "hidden_size": z["width"], "num_hidden_layers": z["layers"], "num_attention_heads": z["heads"],
-                "num_key_value_heads": z["kv_heads"], "head_dim": z["head_dim"], "intermediate_size": z["ff"], "vocab_size": z["vocab"],
-                "max_position_embeddings": 40960, "rms_norm_eps": 1e-6, "rope_theta": 1000000, "tie_word_embeddings": False, "hidden_act": "silu",
-                "attention_bias": False, "torch_dtype": "bfloat16"}
-
+    (new_name, _), (base_name, _) = designs = HYBRID_DESIGNS[args.hybrid_design]
     b, ctx, chunk = args.batch if args.batch != 256 else 64, args.context, 1024
     results = {}
     for name in (args.hybrid_sizes.split(",") if args.hybrid_sizes else HYBRID_SIZES):
         z = HYBRID_SIZES[name]
         results[name] = {}
-        for design, make in (("lamutar", lamutar_cfg), ("qwen3", qwen3_cfg)):
+        for design, make in designs:
             with tempfile.TemporaryDirectory() as d:
                 with open(os.path.join(d, "config.json"), "w") as f:
                     json.dump(make(z), f)
@@ -514,17 +539,19 @@ def hybrid_compare(args):
             runner.exit()
             del runner, driver, seqs
             torch.cuda.empty_cache()
-        lam, q = results[name]["lamutar"], results[name]["qwen3"]
-        results[name]["lamutar_over_qwen3"] = dict(prefill=round(lam["prefill_tok_s"] / q["prefill_tok_s"], 3),
-                                                   decode=round(lam["decode_tok_s"] / q["decode_tok_s"], 3))
-    print(json.dumps(dict(metric="prefill and decode tok/s, Lamutar beside Qwen3 at equal layer sizes (bf16, random weights)",
+        new, base = results[name][new_name], results[name][base_name]
+        results[name][f"{new_name}_over_{base_name}"] = dict(prefill=round(new["prefill_tok_s"] / base["prefill_tok_s"], 3),
+                                                             decode=round(new["decode_tok_s"] / base["decode_tok_s"], 3))
+    print(json.dumps(dict(metric=f"prefill and decode tok/s, {new_name.capitalize()} beside {base_name.capitalize()} at equal layer sizes (bf16, random weights)",
                           batch=b, context=ctx, chunk_tokens=chunk, steps=args.steps, warmup=args.warmup, sizes=results)))
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--hybrid-compare", action="store_true",
-                    help="instead of the headline workload: the Lamutar design beside Qwen3 at equal layer sizes (see hybrid_compare)")
+                    help="instead of the headline workload: a hybrid design beside the closest model at equal layer sizes (see hybrid_compare)")
+    ap.add_argument("--hybrid-design", default="lamutar", choices=sorted(HYBRID_DESIGNS),
+                    help="lamutar (beside Qwen3; the default) or dinatar (beside Lamutar)")
     ap.add_argument("--hybrid-sizes", default="", help="comma-separated subset of " + ",".join(HYBRID_SIZES))
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)

@@ -579,10 +579,14 @@ int32_t nvh_act_mul(const void* x, int64_t row_stride, void* y, int64_t y_stride
 int32_t nvh_logits_scale(const void* logits, int64_t row_stride, float* out, int64_t rows, int64_t vocab, float scale, float cap,
                          int32_t act_f32, nvh_stream_t stream);
 
-/* Linear recurrences with a diagonal decay, state [slots, H, dk, dv] fp32:  S <- diag(w) S + (c k) v^T,  o = S^T q + d v.
+/* Linear recurrences with a diagonal decay, S [dk, dv] per head, stored transposed as state [slots, H, dv, dk] fp32:
+ *   S <- diag(w) S + (c k) v^T,  o = S^T q + d v.
  * nvh_gated_linear_scan: operands fp32; q, k [T, qk_groups, dk] (head h reads group h / (H / qk_groups)), w [T, H, dk] or
  * [T, H] (w_scalar), kscale = c [T, H] (NULL: 1), v [T, H, dv], skip = d [H] (NULL: 0); strides are per token.  Sequences,
- * slots and the fresh start as in nvh_delta_scan; out fp32 [T, H dv].  dk <= 256.
+ * slots and the fresh start as in nvh_delta_scan; out fp32 [T, H dv].  dk <= 256.  segments > 1 (key sizes for which
+ * nvh_scan_segmentable holds; ignored otherwise): a sequence that brings at least segment_min_tokens tokens is cut into that
+ * many segments walked side by side and joined in a second launch; ws_states fp32 [batch, H, segments, dv, dk] and ws_decays
+ * fp32 [batch, H, segments, dk] are scratch.  Results then differ from the unsegmented form within rounding.
  * nvh_hgrn2_prep: q = silu(q), w = f = lower + (1 - lower) sigmoid(f + f_bias), k = 1 - f, v.
  * nvh_gla_prep: q * q_scale, k, v, w = sigmoid(decay_logits)^(1 / tau) (decay_logits fp32).
  * nvh_ssd_conv_prep: the causal convolution (weights [C, taps], last tap on the current token; bias NULL: none) over the
@@ -597,7 +601,9 @@ int32_t nvh_gated_linear_scan(const float* q, int64_t q_stride, const float* k, 
                               int64_t w_stride, int32_t w_scalar, const float* kscale, int64_t kscale_stride, const float* v,
                               int64_t v_stride, const float* skip, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
                               const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
-                              nvh_stream_t stream);
+                              int64_t segments, int64_t segment_min_tokens, float* ws_states, float* ws_decays, nvh_stream_t stream);
+/* Whether key size dk has the segmented form of the scan. */
+int32_t nvh_scan_segmentable(int64_t dk);
 int32_t nvh_hgrn2_prep(const void* q, int64_t q_stride, const void* f, int64_t f_stride, const void* v, int64_t v_stride,
                        const void* f_bias, const void* lower, float* out_q, float* out_k, float* out_w, float* out_v,
                        int64_t num_tokens, int64_t n_k, int64_t n_v, int32_t act_f32, nvh_stream_t stream);
@@ -623,6 +629,11 @@ int32_t nvh_group_rmsnorm_gate(const float* o, const void* weight, int32_t weigh
  * nvh_gemm_any_nt.  nvh_moe_combine: out fp32 [T, dim] = sum_r weights[t, r] y[pos_of_pair[t, r]] (+ shared[t], type A). */
 int32_t nvh_moe_route(const float* logits, int64_t row_stride, int32_t* ids, float* weights, int64_t num_tokens, int64_t experts,
                       int64_t top, nvh_stream_t stream);
+/* nvh_moe_route with the router's product inside: logits = x w^T + bias (x [T, K], w [E, K], bias [E] or NULL, type A;
+ * products and sums in fp32), optionally written to logits_out fp32 [T, E]. */
+int32_t nvh_moe_route_linear(const void* x, int64_t x_row_stride, const void* w, const void* bias, int32_t* ids, float* weights,
+                             float* logits_out, int64_t num_tokens, int64_t experts, int64_t K, int64_t top, int32_t act_f32,
+                             nvh_stream_t stream);
 int64_t nvh_moe_max_tiles(int64_t pairs, int64_t experts);
 int32_t nvh_moe_align(const int32_t* ids, int64_t num_tokens, int64_t experts, int64_t top, int32_t* src_token, int32_t* pos_of_pair,
                       int32_t* tile_expert, int32_t* tile_row0, int32_t* tile_rows, int64_t max_tiles, nvh_stream_t stream);

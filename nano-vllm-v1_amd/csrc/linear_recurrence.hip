@@ -13,6 +13,7 @@
 //                    same bits.
 //   nvh_group_rmsnorm_gate  read-out: RMS norm over groups of columns, weight, and a silu / sigmoid gate before or after.
 // Everything that enters the recurrence is fp32; A (bf16 or fp32) is the type of projections, weights and results.
+#include <algorithm>
 #include "common.h"
 
 namespace {
@@ -105,7 +106,7 @@ __global__ __launch_bounds__(256) void ssd_conv_prep_kernel(SsdPrepArgs p) {
     const bool carried = slot >= 0 && p.context_lens[seq] != hi - lo;       // inputs from before this step exist
     const int C = p.inner + 2 * p.gn, taps = p.taps;
     const float* st = carried ? p.conv_state + (int64_t)slot * (taps - 1) * C : nullptr;
-    for (int c = threadIdx.x; c < C; c += 256) {
+    for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += 256 * gridDim.y) {
         float acc = p.conv_b ? ldf((const A*)p.conv_b, c) : 0.f;
         for (int k = 0; k < taps; ++k) {                     // tap k multiplies the input taps - 1 - k tokens back
             const int back = taps - 1 - k, src = j - back;
@@ -119,6 +120,7 @@ __global__ __launch_bounds__(256) void ssd_conv_prep_kernel(SsdPrepArgs p) {
         else if (c < p.inner + p.gn) p.ok[t * p.gn + (c - p.inner)] = y;
         else p.oq[t * p.gn + (c - p.inner - p.gn)] = y;
     }
+    if (blockIdx.y != 0) return;
     for (int h = threadIdx.x; h < p.H; h += 256) {
         const float dt = softplus_(ldf((const A*)p.dt, t * p.dt_stride + h) + ldf((const A*)p.dt_bias, h));
         p.oc[t * p.H + h] = dt;
@@ -161,16 +163,27 @@ struct ScanArgs {
     const float* v;            // [T, H, dv]
     int64_t v_stride;
     const float* skip;         // [H] or null
-    float* state;              // [slots, H, dk, dv]
+    float* state;              // [slots, H, dv, dk] (the memory S transposed: a column's dk rows are contiguous)
     const int32_t *slots, *cu_seqlens_q, *context_lens;
     float* out;                // [T, H dv]
     int H, dk, dv;
+    int nseg, seg_min;         // segments per long portion (1: none) and the fewest tokens that are cut
+    float *ws_l, *ws_d;        // records of the segments: end states [batch, H, nseg, dv, dk] and decay products [batch, H, nseg, dk]
 };
 
-// Lanes per state column (SUBS), rows held per lane (DKQ), EXACT: dk == DKQ * SUBS (rows DKQ sub .. DKQ sub + DKQ - 1 per
-// lane, read from LDS in 16-byte pieces; otherwise rows SUBS ii + sub, those beyond dk held as zeros).  A workgroup owns
+// Lanes per state column (SUBS), rows held per lane (DKQ), EXACT: dk == DKQ * SUBS (no loop carries a run-time bound; rows
+// beyond dk are held as zeros otherwise).  A workgroup owns
 // COLS = 256 / SUBS columns of one (sequence, head).  A token's staged row: q (dk) | k (dk) | w (dk) | v (COLS) | c | padding.
-template <int DKQ, int SUBS, bool EXACT>
+//
+// MODE 0: a sequence's tokens of this step are walked in one go.
+// MODE 1 and 2, for long portions (a token costs the chain S -> S whatever the chip has idle): the portion is cut into
+// `nseg` segments that are walked side by side.  MODE 1 walks every segment from a zero state (the first from the
+// sequence's state), writes the outputs that this gives, and leaves per segment its end state L_j and the product D_j of
+// its decays.  MODE 2 gives segment j >= 1 what it missed: its true start S_j = D_(j-1) S_(j-1) + L_(j-1), S_1 = L_0,
+// folded from the records, adds (P_t q_t)^T S_j to every output of the segment (P_t: the product of the segment's decays
+// up to t), and the last segment leaves the sequence's state.  Products only, no division: a decay that underflows is a
+// zero.  A sequence with fewer than `seg_min` tokens in the step is one segment (MODE 1 then does all of it).
+template <int DKQ, int SUBS, bool EXACT, int MODE>
 __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
     constexpr int COLS = 256 / SUBS;
     constexpr int CH = (3 * DKQ * SUBS + COLS + 4 + 255) / 256;     // loads per lane and token
@@ -178,17 +191,41 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
     extern __shared__ __attribute__((aligned(16))) float sm[];
     const int seq = blockIdx.x, head = blockIdx.y;
     const int dk = p.dk, dv = p.dv, dkq = (dk + SUBS - 1) / SUBS;
-    const int col0 = blockIdx.z * COLS, lcol = threadIdx.x / SUBS, col = col0 + lcol, sub = threadIdx.x % SUBS;
+    const int seg = MODE == 0 ? 0 : (int)blockIdx.z % p.nseg, colblock = MODE == 0 ? (int)blockIdx.z : (int)blockIdx.z / p.nseg;
+    const int col0 = colblock * COLS, lcol = threadIdx.x / SUBS, col = col0 + lcol, sub = threadIdx.x % SUBS;
     const bool live = col < dv;
-    const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
+    const int seq_lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, seq_hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
     const int slot = p.slots[seq];
-    if (slot < 0 || hi <= lo) return;                        // a padded row (uniform over the workgroup)
-    const bool fresh = p.context_lens[seq] == hi - lo;
-    float* sp = p.state + (((int64_t)slot * p.H + head) * dk) * dv;
-    auto row_of = [&](int ii) { return EXACT ? DKQ * sub + ii : SUBS * ii + sub; };
-    float S[DKQ];
+    if (slot < 0 || seq_hi <= seq_lo) return;                // a padded row (uniform over the workgroup)
+    const int nseg = (MODE != 0 && seq_hi - seq_lo >= p.seg_min) ? p.nseg : 1;
+    if (seg >= nseg || (MODE == 2 && seg == 0)) return;      // (uniform)
+    const int seg_len = (seq_hi - seq_lo + nseg - 1) / nseg;
+    const int lo = seq_lo + seg * seg_len, hi = min(seq_hi, lo + seg_len);   // (hi <= lo: an empty segment; it still leaves its records)
+    const bool fresh = p.context_lens[seq] == seq_hi - seq_lo;
+    float* sp = p.state + (((int64_t)slot * p.H + head) * dv) * dk;      // [dv, dk]: a column's rows lie together
+    const int64_t rec = ((int64_t)seq * p.H + head) * p.nseg;            // this (sequence, head)'s first record
+    // Rows of a lane: with 16-byte LDS reads (EXACT, DKQ a multiple of 4) lane `sub` takes rows 4 sub .. 4 sub + 3 of every 64, so the
+    // 16 lanes of a column read 256 consecutive bytes at a time; otherwise every SUBS-th row, consecutive floats across the lanes.
+    constexpr bool VEC4 = EXACT && DKQ % 4 == 0;
+    auto row_of = [&](int ii) { return VEC4 ? 4 * SUBS * (ii >> 2) + 4 * sub + (ii & 3) : SUBS * ii + sub; };
+    auto row_ok = [&](int ii) { return EXACT || row_of(ii) < dk; };
+    float S[DKQ], P[DKQ];
 #pragma unroll
-    for (int ii = 0; ii < DKQ; ++ii) S[ii] = (live && !fresh && (EXACT || row_of(ii) < dk)) ? sp[(int64_t)row_of(ii) * dv + col] : 0.f;
+    for (int ii = 0; ii < DKQ; ++ii) {
+        P[ii] = 1.f;
+        S[ii] = 0.f;
+        if (MODE != 2 && seg == 0 && live && !fresh && row_ok(ii)) S[ii] = sp[(int64_t)col * dk + row_of(ii)];
+    }
+    if constexpr (MODE == 2) {
+        // the state this segment starts from, folded from the records of the segments before it
+        for (int j = 0; j < seg; ++j) {
+            const float* lj = p.ws_l + ((rec + j) * dv + col) * dk;
+            const float* dj = p.ws_d + (rec + j) * dk;
+#pragma unroll
+            for (int ii = 0; ii < DKQ; ++ii)
+                if (live && row_ok(ii)) S[ii] = __builtin_fmaf(dj[row_of(ii)], S[ii], lj[row_of(ii)]);
+        }
+    }
     const int rowf = (3 * dk + COLS + 4) & ~3;             // (a multiple of 4 floats: rows stay 16-byte aligned)
     const int group = head / (p.H / p.qk_groups);
     const float* qb = p.q + (int64_t)group * dk;
@@ -200,7 +237,8 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
     auto fetch = [&](int t0) {
 #pragma unroll
         for (int tt = 0; tt < TOK; ++tt) {
-            const int64_t tok = min(t0 + tt, hi - 1);
+            const int64_t tok = t0 + tt;
+            if (tok < hi)                                    // (uniform; a one-token step loads one row, not TOK copies of it)
 #pragma unroll
             for (int c = 0; c < CH; ++c) {
                 const int e = min((int)threadIdx.x + 256 * c, rowf - 1);
@@ -214,7 +252,7 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
             }
         }
     };
-    fetch(lo);
+    if (lo < hi) fetch(lo);
     for (int t0 = lo; t0 < hi; t0 += TOK) {
         const int nt = min(TOK, hi - t0);
         __syncthreads();                                     // the previous stage's readers are done
@@ -227,22 +265,22 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
             }
         __syncthreads();
         if (t0 + TOK < hi) fetch(t0 + TOK);
-        for (int tt = 0; tt < nt; ++tt) {
+        // A token's operands are read from LDS one token ahead, into the register set the other token is not using, so the
+        // reads' latency is off the chain S -> S.
+        auto read_token = [&](int tt, float (&xq)[DKQ], float (&xk)[DKQ], float (&xw)[DKQ], float& xv, float& xs) {
             const float* row = sm + tt * rowf;
-            const float xv = row[3 * dk + lcol];
-            const float sv = row[3 * dk + COLS] * xv;
-            float o = 0.f;
-            if constexpr (EXACT && DKQ % 4 == 0) {
+            if constexpr (VEC4) {
 #pragma unroll
                 for (int c4 = 0; c4 < DKQ / 4; ++c4) {
-                    const int i = DKQ * sub + 4 * c4;
-                    const f32x4 vq = *reinterpret_cast<const f32x4*>(row + i), vk = *reinterpret_cast<const f32x4*>(row + dk + i),
-                                vw = *reinterpret_cast<const f32x4*>(row + 2 * dk + i);
+                    const int i = 4 * SUBS * c4 + 4 * sub;
+                    const f32x4 vq = *reinterpret_cast<const f32x4*>(row + i), vw = *reinterpret_cast<const f32x4*>(row + 2 * dk + i);
+                    f32x4 vk = {0.f, 0.f, 0.f, 0.f};
+                    if constexpr (MODE != 2) vk = *reinterpret_cast<const f32x4*>(row + dk + i);
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const float sn = __builtin_fmaf(vw[e], S[4 * c4 + e], vk[e] * sv);
-                        S[4 * c4 + e] = sn;
-                        o = __builtin_fmaf(sn, vq[e], o);
+                        xq[4 * c4 + e] = vq[e];
+                        xk[4 * c4 + e] = vk[e];
+                        xw[4 * c4 + e] = vw[e];
                     }
                 }
             } else {
@@ -251,25 +289,79 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
                     if (EXACT || ii < dkq) {
                         const int i = row_of(ii);
                         const bool in = EXACT || i < dk;     // (a row beyond dk: its state stays zero)
-                        const float xq = in ? row[i] : 0.f, xk = in ? row[dk + i] : 0.f, xw = in ? row[2 * dk + i] : 0.f;
-                        const float sn = __builtin_fmaf(xw, S[ii], xk * sv);
-                        S[ii] = sn;
-                        o = __builtin_fmaf(sn, xq, o);
+                        xq[ii] = in ? row[i] : 0.f;
+                        xk[ii] = in && MODE != 2 ? row[dk + i] : 0.f;
+                        xw[ii] = in ? row[2 * dk + i] : 0.f;
                     }
             }
+            xv = row[3 * dk + lcol];
+            xs = row[3 * dk + COLS];
+        };
+        auto token = [&](int tt, const float (&xq)[DKQ], const float (&xk)[DKQ], const float (&xw)[DKQ], float xv, float xs) {
+            const float sv = xs * xv;
+            float o = 0.f;
+#pragma unroll
+            for (int ii = 0; ii < DKQ; ++ii)
+                if (EXACT || ii < dkq) {
+                    if constexpr (MODE == 2) {
+                        P[ii] *= xw[ii];
+                        o = __builtin_fmaf(P[ii] * xq[ii], S[ii], o);
+                    } else {
+                        const float sn = __builtin_fmaf(xw[ii], S[ii], xk[ii] * sv);
+                        S[ii] = sn;
+                        o = __builtin_fmaf(sn, xq[ii], o);
+                        if constexpr (MODE == 1) P[ii] *= xw[ii];
+                    }
+                }
             if constexpr (SUBS == 16) {
                 o = row16_sum(o);
             } else {
                 o += NVH_DPP(o, 0xB1);
                 o += NVH_DPP(o, 0x4E);
             }
-            if (live && sub == 0) p.out[(int64_t)(t0 + tt) * p.H * dv + head * dv + col] = __builtin_fmaf(skip, xv, o);
+            if (live && sub == 0) {
+                float* dst = p.out + (int64_t)(t0 + tt) * p.H * dv + head * dv + col;
+                if constexpr (MODE == 2) *dst += o;
+                else *dst = __builtin_fmaf(skip, xv, o);
+            }
+        };
+        float cq[DKQ], ck[DKQ], cw[DKQ], cv, cs, nq[DKQ], nk[DKQ], nw[DKQ], nv, ns;
+        read_token(0, cq, ck, cw, cv, cs);
+        int tt = 0;
+        for (; tt + 1 < nt; tt += 2) {
+            read_token(tt + 1, nq, nk, nw, nv, ns);
+            token(tt, cq, ck, cw, cv, cs);
+            read_token(min(tt + 2, TOK - 1), cq, ck, cw, cv, cs);
+            token(tt + 1, nq, nk, nw, nv, ns);
         }
+        if (tt < nt) token(tt, cq, ck, cw, cv, cs);
+    }
+    if constexpr (MODE == 2) {
+        if (seg != nseg - 1) return;
+        // the last segment: the sequence's state after this step, D S + L with its own record
+        const float* lj = p.ws_l + ((rec + seg) * dv + col) * dk;
+#pragma unroll
+        for (int ii = 0; ii < DKQ; ++ii)
+            if (live && row_ok(ii)) S[ii] = __builtin_fmaf(P[ii], S[ii], lj[row_of(ii)]);
+    }
+    if (MODE == 1 && nseg > 1) {
+        if (live) {
+            float* lj = p.ws_l + ((rec + seg) * dv + col) * dk;
+#pragma unroll
+            for (int ii = 0; ii < DKQ; ++ii)
+                if (row_ok(ii)) lj[row_of(ii)] = S[ii];
+        }
+        if (colblock == 0 && lcol == 0) {
+#pragma unroll
+            for (int ii = 0; ii < DKQ; ++ii)
+                if (row_ok(ii)) p.ws_d[(rec + seg) * dk + row_of(ii)] = P[ii];
+        }
+        return;
     }
     if (live) {
 #pragma unroll
         for (int ii = 0; ii < DKQ; ++ii)
-            if (EXACT || row_of(ii) < dk) sp[(int64_t)row_of(ii) * dv + col] = S[ii];
+            if (row_ok(ii)) sp[(int64_t)col * dk + row_of(ii)] = S[ii];
     }
 }
 
@@ -305,14 +397,62 @@ __global__ __launch_bounds__(256) void group_rmsnorm_gate_kernel(const float* __
     }
 }
 
+// The same with one workgroup per (token, group), for groups of more than 256 columns (up to 256 PER): the gated values stay
+// in registers between the sum and the write.
+template <typename A, int PER>
+__global__ __launch_bounds__(256) void group_rmsnorm_gate_block_kernel(const float* __restrict__ o, const A* __restrict__ weight, int w_full, const A* __restrict__ gate,
+                                                                       int64_t gate_stride, int gate_act, int gate_first, A* __restrict__ y, int64_t y_stride,
+                                                                       int groups, int gs, float eps) {
+    __shared__ float red[4];
+    const int64_t t = blockIdx.x / groups;
+    const int g = (int)(blockIdx.x - t * groups);
+    const float* orow = o + (t * groups + g) * gs;
+    const A* grow = gate ? gate + t * gate_stride + (int64_t)g * gs : nullptr;
+    const bool pre = gate && gate_act && gate_first, post = gate && gate_act && !gate_first;
+    float v[PER], gv[PER], ss = 0.f;
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        v[j] = i < gs ? orow[i] : 0.f;
+        gv[j] = 1.f;
+        if (grow && gate_act && i < gs) {
+            const float z = (float)grow[i];
+            gv[j] = gate_act == 1 ? sigmoid_(z) : silu_(z);
+        }
+        if (pre) v[j] *= gv[j];
+        ss += v[j] * v[j];
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float inv = 1.0f / sqrtf((red[0] + red[1] + red[2] + red[3]) / (float)gs + eps);
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+        const int i = threadIdx.x + 256 * j;
+        if (i < gs) {
+            float r = v[j] * inv * ldf(weight, w_full ? (int64_t)g * gs + i : i);
+            if (post) r *= gv[j];
+            y[t * y_stride + (int64_t)g * gs + i] = (A)r;
+        }
+    }
+}
+
 template <int DKQ, int SUBS, bool EXACT>
 void launch_scan_as(const ScanArgs& p, int64_t batch, hipStream_t st) {
     constexpr int COLS = 256 / SUBS;
     constexpr int CH = (3 * DKQ * SUBS + COLS + 4 + 255) / 256;
     constexpr int TOK = (32 / CH) < 2 ? 2 : (32 / CH);
-    const dim3 grid((unsigned)batch, (unsigned)p.H, (unsigned)nvh_cdiv(p.dv, COLS));
+    const unsigned colblocks = (unsigned)nvh_cdiv(p.dv, COLS);
     const size_t lds = sizeof(float) * (size_t)TOK * ((3 * p.dk + COLS + 4) & ~3);
-    gated_linear_scan_kernel<DKQ, SUBS, EXACT><<<grid, 256, lds, st>>>(p);
+    if constexpr (EXACT) {
+        if (p.nseg > 1) {
+            const dim3 grid((unsigned)batch, (unsigned)p.H, colblocks * (unsigned)p.nseg);
+            gated_linear_scan_kernel<DKQ, SUBS, EXACT, 1><<<grid, 256, lds, st>>>(p);
+            gated_linear_scan_kernel<DKQ, SUBS, EXACT, 2><<<grid, 256, lds, st>>>(p);
+            return;
+        }
+    }
+    gated_linear_scan_kernel<DKQ, SUBS, EXACT, 0><<<dim3((unsigned)batch, (unsigned)p.H, colblocks), 256, lds, st>>>(p);
 }
 
 }  // namespace
@@ -368,8 +508,10 @@ extern "C" int32_t nvh_ssd_conv_prep(const void* xbc, int64_t xbc_stride, const 
     if (num_tokens == 0 || batch == 0) return NVH_OK;
     p.ov = out_x, p.ok = out_b, p.oq = out_c, p.oc = out_dt, p.ow = out_decay;
     hipStream_t st = (hipStream_t)stream;
-    if (act_f32) ssd_conv_prep_kernel<float><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
-    else ssd_conv_prep_kernel<bf16><<<dim3((unsigned)num_tokens), 256, 0, st>>>(p);
+    // few tokens: the channels are spread over more workgroups (a token's row is short work for one)
+    const dim3 grid((unsigned)num_tokens, (unsigned)(num_tokens >= 512 ? 1 : std::min<int64_t>(nvh_cdiv(inner + 2 * gn, 256), 16)));
+    if (act_f32) ssd_conv_prep_kernel<float><<<grid, 256, 0, st>>>(p);
+    else ssd_conv_prep_kernel<bf16><<<grid, 256, 0, st>>>(p);
     NVH_CHECK_LAUNCH("nvh_ssd_conv_prep");
     return NVH_OK;
 }
@@ -390,17 +532,27 @@ extern "C" int32_t nvh_conv_state_update(const void* xbc, int64_t xbc_stride, fl
     return NVH_OK;
 }
 
+// Key sizes whose scan has the segmented form (the exact instantiations below).
+extern "C" int32_t nvh_scan_segmentable(int64_t dk) {
+    return dk % 16 == 0 && (dk / 16 <= 4 || dk / 16 == 6 || dk / 16 == 8 || dk / 16 == 16);
+}
+
 extern "C" int32_t nvh_gated_linear_scan(const float* q, int64_t q_stride, const float* k, int64_t k_stride, int64_t qk_groups, const float* w,
                                          int64_t w_stride, int32_t w_scalar, const float* kscale, int64_t kscale_stride, const float* v,
                                          int64_t v_stride, const float* skip, float* state, const int32_t* slots, const int32_t* cu_seqlens_q,
                                          const int32_t* context_lens, float* out, int64_t batch, int64_t heads, int64_t dk, int64_t dv,
-                                         nvh_stream_t stream) {
+                                         int64_t segments, int64_t segment_min_tokens, float* ws_states, float* ws_decays, nvh_stream_t stream) {
     NVH_REQUIRE(q && k && w && v && state && slots && context_lens && out, NVH_EINVAL, "nvh_gated_linear_scan: null pointer");
     NVH_REQUIRE(batch >= 0 && heads > 0 && dk > 0 && dv > 0 && qk_groups > 0 && heads % qk_groups == 0, NVH_EINVAL, "nvh_gated_linear_scan: bad sizes");
     NVH_REQUIRE(dk <= 256, NVH_ENOSYS, "nvh_gated_linear_scan: key size %ld above 256", (long)dk);
     if (batch == 0) return NVH_OK;
-    const ScanArgs p{q, k, q_stride, k_stride, (int)qk_groups, w, w_stride, w_scalar, kscale, kscale_stride, v, v_stride, skip, state, slots,
-                     cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dv};
+    ScanArgs p{q, k, q_stride, k_stride, (int)qk_groups, w, w_stride, w_scalar, kscale, kscale_stride, v, v_stride, skip, state, slots,
+                     cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dv, 1, 1 << 30, ws_states, ws_decays};
+    if (segments > 1 && nvh_scan_segmentable(dk)) {
+        NVH_REQUIRE(segments <= 64 && segment_min_tokens >= 2 * segments && ws_states && ws_decays && cu_seqlens_q, NVH_EINVAL, "nvh_gated_linear_scan: bad segments");
+        p.nseg = (int)segments;
+        p.seg_min = (int)segment_min_tokens;
+    }
     hipStream_t st = (hipStream_t)stream;
     // (the choice depends on dk alone, so a sequence sees one summation order whatever the batch or the cut)
     if (dk % 16 == 0) {
@@ -433,8 +585,23 @@ extern "C" int32_t nvh_group_rmsnorm_gate(const float* o, const void* weight, in
     NVH_REQUIRE(o && weight && y && rows >= 0 && groups > 0 && group_size > 0 && gate_act >= 0 && gate_act <= 2 && (!gate_act || gate), NVH_EINVAL,
                 "nvh_group_rmsnorm_gate: bad argument");
     if (rows == 0) return NVH_OK;
-    const unsigned blocks = (unsigned)nvh_cdiv(rows * groups, 4);
     hipStream_t st = (hipStream_t)stream;
+    // (the form depends on the group size alone: a row sees one summation order whatever the batch or the cut)
+    if (group_size > 256 && group_size <= 8192 && rows * groups < (1ll << 31)) {
+        const dim3 grid((unsigned)(rows * groups));
+#define NVH_GN_BLOCK(A, PER) group_rmsnorm_gate_block_kernel<A, PER><<<grid, 256, 0, st>>>(o, (const A*)weight, weight_full, (const A*)gate, gate_stride, gate_act, gate_first, (A*)y, y_stride, (int)groups, (int)group_size, eps)
+        if (group_size <= 2048) {
+            if (act_f32) NVH_GN_BLOCK(float, 8);
+            else NVH_GN_BLOCK(bf16, 8);
+        } else {
+            if (act_f32) NVH_GN_BLOCK(float, 32);
+            else NVH_GN_BLOCK(bf16, 32);
+        }
+#undef NVH_GN_BLOCK
+        NVH_CHECK_LAUNCH("nvh_group_rmsnorm_gate");
+        return NVH_OK;
+    }
+    const unsigned blocks = (unsigned)nvh_cdiv(rows * groups, 4);
     if (act_f32) group_rmsnorm_gate_kernel<float><<<dim3(blocks), 256, 0, st>>>(o, (const float*)weight, weight_full, (const float*)gate, gate_stride, gate_act, gate_first, (float*)y, y_stride, rows, (int)groups, (int)group_size, eps);
     else group_rmsnorm_gate_kernel<bf16><<<dim3(blocks), 256, 0, st>>>(o, (const bf16*)weight, weight_full, (const bf16*)gate, gate_stride, gate_act, gate_first, (bf16*)y, y_stride, rows, (int)groups, (int)group_size, eps);
     NVH_CHECK_LAUNCH("nvh_group_rmsnorm_gate");

@@ -1,6 +1,7 @@
 // Mixture of experts: a token goes to the `top` experts whose router logits are largest, mixed with the weights that a
 // softmax over just these `top` logits gives.
-//   nvh_moe_route     fp32 router logits [T, E] -> expert ids and weights [T, top] (ties go to the lower expert id)
+//   nvh_moe_route     fp32 router logits [T, E] -> expert ids and weights [T, top] (ties go to the lower expert id);
+//                     nvh_moe_route_linear forms the logits itself (x W^T + b in fp32) in the same launch
 //   nvh_moe_align     the (token, choice) pairs ordered by expert: for every position in that order the token it comes
 //                     from, for every pair its position, and a list of 64-row tiles (expert, first position, rows) that
 //                     covers every expert's block - all on the device, so a step never waits for the host and the whole
@@ -59,6 +60,105 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 #pragma unroll
         for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
             if (lane + 64 * j == be) z[j] = -INFINITY;       // taken
+    }
+    if (lane == 0)
+        for (int r = 0; r < top; ++r) weights[t * top + r] = weights[t * top + r] / denom;
+}
+
+// The same with the router's product inside: z[e] = x . w[e] + bias[e] in fp32, every expert's dot product spread over the
+// wave's lanes (lane l takes elements l, l + 64, ... of the row) and summed across it.
+// Eight consecutive elements p[off .. off + 7] as floats; those at or beyond `valid` read as zero.  `vec`: 16-byte accesses are allowed.
+template <typename A>
+__device__ __forceinline__ void load8(const A* p, int64_t off, int valid, bool vec, float (&out)[8]) {
+    if (vec && valid >= 8) {
+        if constexpr (sizeof(A) == 2) {
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(p + off);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) out[i] = (float)v[i];
+        } else {
+            const f32x4 a = *reinterpret_cast<const f32x4*>(p + off), b = *reinterpret_cast<const f32x4*>(p + off + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                out[i] = a[i];
+                out[4 + i] = b[i];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = i < valid ? (float)p[off + i] : 0.f;
+    }
+}
+
+template <typename A>
+__global__ __launch_bounds__(256) void moe_route_linear_kernel(const A* __restrict__ x, int64_t ldx, const A* __restrict__ w, const A* __restrict__ bias,
+                                                               int32_t* __restrict__ ids, float* __restrict__ weights, float* __restrict__ logits_out,
+                                                               int64_t tokens, int experts, int K, int top, int vec) {
+    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (t >= tokens) return;
+    const int lane = threadIdx.x & 63;
+    const A* xr = x + t * ldx;
+    float z[ROUTE_MAX_PER_LANE];
+#pragma unroll
+    for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) z[j] = -INFINITY;
+    // eight experts at a time: their loads do not wait for one another; a lane takes 8 consecutive elements of every 512
+    constexpr int EG = 8;
+    for (int e0 = 0; e0 < experts; e0 += EG) {
+        float acc[EG];
+#pragma unroll
+        for (int g = 0; g < EG; ++g) acc[g] = 0.f;
+        for (int k0 = lane * 8; k0 < K; k0 += 512) {
+            float xv[8];
+            load8(xr, k0, K - k0, vec, xv);
+#pragma unroll
+            for (int g = 0; g < EG; ++g) {
+                float wv[8];
+                load8(w + (int64_t)min(e0 + g, experts - 1) * K, k0, K - k0, vec, wv);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[g] = __builtin_fmaf(xv[i], wv[i], acc[g]);
+            }
+        }
+#pragma unroll
+        for (int g = 0; g < EG; ++g) {
+            const int e = e0 + g;
+            if (e >= experts) break;
+            const float s = wave_sum(acc[g]) + (bias ? (float)bias[e] : 0.f);
+            if (logits_out && lane == 0) logits_out[t * experts + e] = s;
+#pragma unroll
+            for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
+                if (lane + 64 * j == e) z[j] = s;
+        }
+    }
+    float first = 0.f, denom = 0.f;
+    for (int r = 0; r < top; ++r) {
+        float bv = -INFINITY;
+        int be = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) {
+            const int e = lane + 64 * j;
+            if (z[j] > bv || (z[j] == bv && e < be && z[j] != -INFINITY)) {
+                bv = z[j];
+                be = e;
+            }
+        }
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const float ov = __shfl_xor(bv, off, 64);
+            const int oe = __shfl_xor(be, off, 64);
+            if (ov > bv || (ov == bv && oe < be)) {
+                bv = ov;
+                be = oe;
+            }
+        }
+        if (r == 0) first = bv;
+        const float wgt = expf(bv - first);
+        denom += wgt;
+        if (lane == 0) {
+            ids[t * top + r] = be;
+            weights[t * top + r] = wgt;
+        }
+#pragma unroll
+        for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
+            if (lane + 64 * j == be) z[j] = -INFINITY;
     }
     if (lane == 0)
         for (int r = 0; r < top; ++r) weights[t * top + r] = weights[t * top + r] / denom;
@@ -167,6 +267,22 @@ extern "C" int32_t nvh_moe_route(const float* logits, int64_t row_stride, int32_
     if (num_tokens == 0) return NVH_OK;
     moe_route_kernel<<<dim3((unsigned)nvh_cdiv(num_tokens, 4)), 256, 0, (hipStream_t)stream>>>(logits, row_stride, ids, weights, num_tokens, (int)experts, (int)top);
     NVH_CHECK_LAUNCH("nvh_moe_route");
+    return NVH_OK;
+}
+
+extern "C" int32_t nvh_moe_route_linear(const void* x, int64_t x_row_stride, const void* w, const void* bias, int32_t* ids, float* weights,
+                                        float* logits_out, int64_t num_tokens, int64_t experts, int64_t K, int64_t top, int32_t act_f32,
+                                        nvh_stream_t stream) {
+    NVH_REQUIRE(x && w && ids && weights, NVH_EINVAL, "nvh_moe_route_linear: null pointer");
+    NVH_REQUIRE(num_tokens >= 0 && experts > 0 && top > 0 && top <= experts && K > 0 && K < (1 << 30) && x_row_stride >= K, NVH_EINVAL, "nvh_moe_route_linear: bad sizes");
+    NVH_REQUIRE(experts <= 64 * ROUTE_MAX_PER_LANE, NVH_ENOSYS, "nvh_moe_route_linear: %ld experts above %d", (long)experts, 64 * ROUTE_MAX_PER_LANE);
+    if (num_tokens == 0) return NVH_OK;
+    const dim3 grid((unsigned)nvh_cdiv(num_tokens, 4));
+    hipStream_t st = (hipStream_t)stream;
+    const int vec = K % 8 == 0 && x_row_stride % 8 == 0 && nvh_aligned16(x) && nvh_aligned16(w);
+    if (act_f32) moe_route_linear_kernel<float><<<grid, 256, 0, st>>>((const float*)x, x_row_stride, (const float*)w, (const float*)bias, ids, weights, logits_out, num_tokens, (int)experts, (int)K, (int)top, vec);
+    else moe_route_linear_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, x_row_stride, (const bf16*)w, (const bf16*)bias, ids, weights, logits_out, num_tokens, (int)experts, (int)K, (int)top, vec);
+    NVH_CHECK_LAUNCH("nvh_moe_route_linear");
     return NVH_OK;
 }
 

@@ -108,7 +108,8 @@ SIGNATURES = {
     "nvh_act_mul": (i32, [vp, i64, vp, i64, i64, i64, i32, i32, i32, vp]),
     "nvh_logits_scale": (i32, [vp, i64, vp, i64, i64, f32, f32, i32, vp]),
     # linear recurrences with a diagonal decay (csrc/linear_recurrence.hip)
-    "nvh_gated_linear_scan": (i32, [vp, i64, vp, i64, i64, vp, i64, i32, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, vp]),
+    "nvh_gated_linear_scan": (i32, [vp, i64, vp, i64, i64, vp, i64, i32, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, vp]),
+    "nvh_scan_segmentable": (i32, [i64]),
     "nvh_hgrn2_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, i64, i64, i64, i32, vp]),
     "nvh_gla_prep": (i32, [vp, i64, vp, i64, vp, i64, vp, i64, f32, f32, vp, vp, vp, vp, i64, i64, i64, i32, vp]),
     "nvh_ssd_conv_prep": (i32, [vp, i64, vp, i64, vp, vp, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, vp, vp, vp, vp, vp, i32, vp]),
@@ -116,6 +117,7 @@ SIGNATURES = {
     "nvh_group_rmsnorm_gate": (i32, [vp, vp, i32, vp, i64, i32, i32, vp, i64, i64, i64, i64, f32, i32, vp]),
     # mixture of experts (csrc/moe.hip)
     "nvh_moe_route": (i32, [vp, i64, vp, vp, i64, i64, i64, vp]),
+    "nvh_moe_route_linear": (i32, [vp, i64, vp, vp, vp, vp, vp, i64, i64, i64, i64, i32, vp]),
     "nvh_moe_max_tiles": (i64, [i64, i64]),
     "nvh_moe_align": (i32, [vp, i64, i64, i64, vp, vp, vp, vp, vp, i64, vp]),
     "nvh_gemm_grouped_any_nt": (i32, [vp, i64, vp, vp, vp, i64, vp, vp, vp, i64, i64, i64, i32, i32, vp]),

@@ -267,7 +267,7 @@ class ModelRunner:
                           file=sys.stderr)
                     self.graphs, self.graph_bs, self.enforce_eager = {}, [], True
         finally:
-            torch.set_default_device("cpu")
+            torch.set_default_device(None)          # (not "cpu": a default device of any name keeps a Python hook on every torch call)
             torch.set_default_dtype(prev_dtype)
 
         if self.world_size > 1 and not self.external_group:

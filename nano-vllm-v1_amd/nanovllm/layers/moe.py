@@ -58,7 +58,7 @@ class SparseMoE(nn.Module):
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         """x [T, width] in the activation type -> fp32 [T, width]."""
-        ids, weights = ops.moe_route(self.router(x, out_f32=True), self.top)
+        ids, weights = ops.moe_route_linear(x, self.router.weight.data, None if self.router.bias is None else self.router.bias.data, self.top)
         plan = ops.moe_align(ids, self.experts)
         hidden = ops.act_mul(ops.linear_grouped(x, self.gate_up.data, plan, gather=True), self.act, True)
         y = ops.linear_grouped(hidden, self.down.data, plan, gather=False)

@@ -83,14 +83,14 @@ class DiagonalDecayRecurrence(_StatePool):
     starts in this step (kernel: nvh_gated_linear_scan, csrc/linear_recurrence.hip)."""
 
     def __init__(self, num_heads: int, key_dim: int, value_dim: int, qk_groups: int | None = None, state_runs: int = 1):
-        super().__init__((num_heads, key_dim, value_dim), state_runs)
+        super().__init__((num_heads, value_dim, key_dim), state_runs)      # stored transposed: a column's key rows lie together
         self.num_heads, self.key_dim, self.value_dim, self.qk_groups = num_heads, key_dim, value_dim, qk_groups or num_heads
 
     def forward(self, q, k, w, v, run: int = 0, kscale=None, skip=None) -> torch.Tensor:
         state = self.pool(run)
         ctx = get_context()
         return ops.gated_linear_scan(q, k, w, v, state, ctx.state_slots, ctx.cu_seqlens_q, ctx.context_lens, self.num_heads, self.key_dim,
-                                     self.value_dim, self.qk_groups, kscale, skip)
+                                     self.value_dim, self.qk_groups, kscale, skip, max_seqlen_q=ctx.max_seqlen_q or 0)
 
 
 class HGRN2(nn.Module):

@@ -794,11 +794,16 @@ def _f32_rows(t, *tensors):
         assert x.dtype == F32 and x.is_cuda and x.stride(-1) == 1 and x.shape[0] == t
 
 
+SCAN_SEGMENT_MIN_TOKENS = 256      # a sequence that brings at least this many tokens to a step is scanned in segments ...
+SCAN_SEGMENT_MAX_BATCH = 8         # ... in steps of at most this many sequences (the segments' records are scratch per sequence)
+
+
 def gated_linear_scan(q, k, w, v, state, slots, cu_seqlens_q, context_lens, heads: int, dk: int, dv: int, qk_groups: int | None = None,
-                      kscale=None, skip=None) -> torch.Tensor:
+                      kscale=None, skip=None, max_seqlen_q: int = 0) -> torch.Tensor:
     """S <- diag(w) S + (kscale k) v^T, o = S^T q + skip v over the packed tokens; fp32 operands q, k [T, qk_groups * dk],
     w [T, H * dk] or [T, H] (one decay per head), kscale [T, H] | None, v [T, H * dv], skip [H] | None; `state`
-    [slots, H, dk, dv] fp32 is read (unless the sequence starts in this step) and left updated.  Returns fp32 [T, H * dv]."""
+    [slots, H, dv, dk] fp32 (S transposed: a column's rows lie together) is read (unless the sequence starts in this step) and
+    left updated.  Returns fp32 [T, H * dv]."""
     t = v.shape[0]
     g = qk_groups or heads
     _f32_rows(t, q, k, w, v)
@@ -806,14 +811,23 @@ def gated_linear_scan(q, k, w, v, state, slots, cu_seqlens_q, context_lens, head
     w_scalar = w.shape[1] == heads and dk != 1
     assert kscale is None or (kscale.dtype == F32 and kscale.shape == (t, heads) and kscale.stride(1) == 1)
     assert skip is None or (skip.dtype == F32 and skip.numel() == heads and skip.is_contiguous())
-    assert state.dtype == F32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dk, dv) and slots.dtype == torch.int32
+    assert state.dtype == F32 and state.is_contiguous() and tuple(state.shape[1:]) == (heads, dv, dk) and slots.dtype == torch.int32
     assert context_lens.dtype == torch.int32 and (cu_seqlens_q is None or cu_seqlens_q.dtype == torch.int32)
     batch = context_lens.numel()
     assert cu_seqlens_q is not None or t == batch
     out = torch.empty(t, heads * dv, dtype=F32, device=v.device)
+    # Long portions (prompt chunks) in small batches: segments walked side by side, joined in a second launch.  The choice
+    # depends on the step's longest portion, so a position's result may differ between schedules - within fp32 rounding.
+    segments, ws_l, ws_d = 1, None, None
+    if (cu_seqlens_q is not None and batch <= SCAN_SEGMENT_MAX_BATCH and max_seqlen_q >= SCAN_SEGMENT_MIN_TOKENS
+            and _hip.lib().nvh_scan_segmentable(dk)):
+        segments = 8 if max_seqlen_q >= 2 * SCAN_SEGMENT_MIN_TOKENS else 4
+        ws_l = torch.empty(batch * heads * segments * dv * dk, dtype=F32, device=v.device)
+        ws_d = torch.empty(batch * heads * segments * dk, dtype=F32, device=v.device)
     _hip.call("nvh_gated_linear_scan", q.data_ptr(), q.stride(0), k.data_ptr(), k.stride(0), g, w.data_ptr(), w.stride(0), int(w_scalar),
               _p(kscale), kscale.stride(0) if kscale is not None else 0, v.data_ptr(), v.stride(0), _p(skip), state.data_ptr(), slots.data_ptr(),
-              _p(cu_seqlens_q), context_lens.data_ptr(), out.data_ptr(), batch, heads, dk, dv, _stream())
+              _p(cu_seqlens_q), context_lens.data_ptr(), out.data_ptr(), batch, heads, dk, dv, segments, SCAN_SEGMENT_MIN_TOKENS, _p(ws_l), _p(ws_d),
+              _stream())
     return out
 
 
@@ -889,6 +903,19 @@ def moe_route(logits: torch.Tensor, top: int):
     weights = torch.empty(t, top, dtype=F32, device=logits.device)
     _hip.call("nvh_moe_route", logits.data_ptr(), logits.stride(0), ids.data_ptr(), weights.data_ptr(), t, e, top, _stream())
     return ids, weights
+
+
+def moe_route_linear(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor | None, top: int, want_logits: bool = False):
+    """moe_route of the fp32 logits x @ weight^T + bias, formed inside the same launch: (ids, weights[, logits])."""
+    f = _act_flag(x, weight) if bias is None else _act_flag(x, weight, bias)
+    t, k = x.shape
+    e = weight.shape[0]
+    assert x.stride(1) == 1 and weight.is_contiguous() and weight.shape[1] == k and (bias is None or bias.numel() == e)
+    ids = torch.empty(t, top, dtype=torch.int32, device=x.device)
+    weights = torch.empty(t, top, dtype=F32, device=x.device)
+    logits = torch.empty(t, e, dtype=F32, device=x.device) if want_logits else None
+    _hip.call("nvh_moe_route_linear", x.data_ptr(), x.stride(0), weight.data_ptr(), _p(bias), ids.data_ptr(), weights.data_ptr(), _p(logits), t, e, k, top, f, _stream())
+    return (ids, weights, logits) if want_logits else (ids, weights)
 
 
 def moe_align(ids: torch.Tensor, experts: int) -> dict:

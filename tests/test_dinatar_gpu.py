@@ -253,11 +253,14 @@ def test_scan_against_the_recurrence_written_out():
     are and are not multiples of 16 and of 4; two sequences, one continued from a state, one fresh, in slots out of order."""
     from nanovllm import ops
     g = torch.Generator().manual_seed(0)
-    for H, G, dk, dv, scalar in [(4, 2, 20, 12, True), (2, 2, 16, 48, False), (3, 1, 64, 70, True), (2, 2, 37, 5, False), (1, 1, 128, 64, False)]:
-        lens, past = [9, 5], [4, 0]
+    for H, G, dk, dv, scalar, lens in [(4, 2, 20, 12, True, [9, 5]), (2, 2, 16, 48, False, [9, 5]), (3, 1, 64, 70, True, [9, 5]), (2, 2, 37, 5, False, [9, 5]),
+                                       (1, 1, 128, 64, False, [9, 5]),
+                                       # long portions: walked in segments that are joined afterwards (beside a short one that is not)
+                                       (2, 1, 32, 24, True, [300, 7]), (1, 1, 64, 16, False, [1, 555]), (2, 2, 16, 8, False, [256, 257])]:
+        past = [4, 0]
         T = sum(lens)
         q, k = torch.randn(T, G * dk, generator=g), torch.randn(T, G * dk, generator=g)
-        w = torch.rand(T, H if scalar else H * dk, generator=g)
+        w = torch.rand(T, H if scalar else H * dk, generator=g) ** (0.02 if max(lens) > 100 else 1.0)     # (long runs: decays near one, so far tokens count)
         c = torch.rand(T, H, generator=g) + 0.5
         v = torch.randn(T, H * dv, generator=g)
         d = torch.randn(H, generator=g)
@@ -275,13 +278,13 @@ def test_scan_against_the_recurrence_written_out():
                     want[t, h * dv:(h + 1) * dv] = S.T @ q[t, gq * dk:(gq + 1) * dk].double() + d[h].double() * v[t, h * dv:(h + 1) * dv].double()
                 new_state[slots[b], h] = S
             t0 += n
-        st = state.cuda()
+        st = state.transpose(2, 3).contiguous().cuda()          # the pool holds S transposed: [slots, H, dv, dk]
         cu = torch.tensor([0, lens[0], T], dtype=torch.int32).cuda()
         ctx = torch.tensor([lens[0] + past[0], lens[1] + past[1]], dtype=torch.int32).cuda()
         got = ops.gated_linear_scan(q.cuda(), k.cuda(), w.cuda(), v.cuda(), st, torch.tensor(slots, dtype=torch.int32).cuda(), cu, ctx, H, dk, dv, G,
-                                    kscale=c.cuda(), skip=d.cuda())
+                                    kscale=c.cuda(), skip=d.cuda(), max_seqlen_q=max(lens))
         assert (got.cpu().double() - want).abs().max() < 1e-4 * max(1.0, float(want.abs().max())), (H, G, dk, dv)
-        assert (st.cpu().double() - new_state).abs().max() < 1e-4 * max(1.0, float(new_state.abs().max()))
+        assert (st.cpu().double().transpose(2, 3) - new_state).abs().max() < 1e-4 * max(1.0, float(new_state.abs().max()))
 
 
 def test_router_picks_the_largest_and_weighs_them_alone():
@@ -293,6 +296,15 @@ def test_router_picks_the_largest_and_weighs_them_alone():
         val, idx = torch.topk(z, top, dim=-1)
         assert torch.equal(ids.cpu().long(), idx)
         assert (wts.cpu() - torch.softmax(val, -1)).abs().max() < 1e-6
+        # the router's product inside the same launch, both activation types
+        x, w, b = torch.randn(33, 70, generator=g), torch.randn(E, 70, generator=g), torch.randn(E, generator=g)
+        for cast in (torch.float32, torch.bfloat16):
+            xa, wa, ba = x.to(cast), w.to(cast), b.to(cast)
+            zz = xa.double() @ wa.double().T + ba.double()
+            ids, wts, lg = ops.moe_route_linear(xa.cuda(), wa.cuda(), ba.cuda(), top, want_logits=True)
+            assert (lg.cpu().double() - zz).abs().max() < 1e-4
+            val, idx = torch.topk(lg.cpu(), top, dim=-1)
+            assert torch.equal(ids.cpu().long(), idx) and (wts.cpu() - torch.softmax(val, -1)).abs().max() < 1e-6
     z = torch.tensor([[1.0, 3.0, 3.0, 0.0]])
     ids, _ = ops.moe_route(z.cuda(), 2)
     assert ids.cpu().tolist() == [[1, 2]]                     # a tie: the lower expert first
@@ -340,6 +352,24 @@ def test_layer_close_kernel_against_its_formula():
         xg = x.cuda()
         h = ops.residual_norm(xg, a=a.cuda(), norm="rms", weight=nw.cuda(), eps=1e-6)
         assert (h.cpu() - unit(x + a) * nw).abs().max() < 1e-4 and (xg.cpu() - (x + a)).abs().max() < 1e-6
+
+
+def test_grouped_norm_with_gates_before_and_after():
+    """Groups small (a wave each) and large (a workgroup each), a weight per group or per column, silu gate first, sigmoid gate last."""
+    from nanovllm import ops
+    g = torch.Generator().manual_seed(4)
+    unit = lambda v: v / torch.sqrt((v * v).mean(-1, keepdim=True) + 1e-5)
+    for groups, gs in [(3, 20), (2, 64), (1, 600), (2, 2048), (1, 2500)]:
+        o, gate = torch.randn(7, groups * gs, generator=g), torch.randn(7, 2 * groups * gs, generator=g)[:, groups * gs:]
+        for w in (torch.randn(gs, generator=g), torch.randn(groups * gs, generator=g)):
+            wf = (w if w.numel() == groups * gs else w.repeat(groups))
+            first = (unit((o * torch.nn.functional.silu(gate)).view(7, groups, gs)).reshape(7, -1) * wf)
+            last = unit(o.view(7, groups, gs)).reshape(7, -1) * wf * torch.sigmoid(gate)
+            plain = unit(o.view(7, groups, gs)).reshape(7, -1) * wf
+            gc = gate.cuda()
+            assert (ops.group_rmsnorm_gate(o.cuda(), w.cuda(), gs, 1e-5, gc, "silu", gate_first=True).cpu() - first).abs().max() < 1e-4
+            assert (ops.group_rmsnorm_gate(o.cuda(), w.cuda(), gs, 1e-5, gc, "sigmoid", gate_first=False).cpu() - last).abs().max() < 1e-4
+            assert (ops.group_rmsnorm_gate(o.cuda(), w.cuda(), gs, 1e-5).cpu() - plain).abs().max() < 1e-4
 
 
 # ----------------------------------------------------------------------------------------------------- schedules
@@ -541,6 +571,8 @@ def test_recurrent_states_carry_a_token_from_far_back(tmp_path):
         rp = case.replay("float32", max_tokens=1024)
         try:
             run_schedule(rp, case, {"a": toks}, [[("a", 100)], [("a", 156)], [("a", 1)], [("a", 140)], [("a", 2)], [("a", 1)]], "float32")
+            # portions long enough to be scanned in segments, beside a short request; then the state they left is decoded from
+            run_schedule(rp, case, {"b": toks, "c": toks[:9]}, [[("b", 290), ("c", 8)], [("b", 109), ("c", 1)], [("b", 1)]], "float32")
         finally:
             rp.close()
 
