@@ -227,6 +227,7 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
         }
     }
     const int rowf = (3 * dk + COLS + 4) & ~3;             // (a multiple of 4 floats: rows stay 16-byte aligned)
+    float* osm = sm + TOK * rowf;                            // [TOK][COLS]: the stage's outputs
     const int group = head / (p.H / p.qk_groups);
     const float* qb = p.q + (int64_t)group * dk;
     const float* kb = p.k + (int64_t)group * dk;
@@ -319,11 +320,7 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
                 o += NVH_DPP(o, 0xB1);
                 o += NVH_DPP(o, 0x4E);
             }
-            if (live && sub == 0) {
-                float* dst = p.out + (int64_t)(t0 + tt) * p.H * dv + head * dv + col;
-                if constexpr (MODE == 2) *dst += o;
-                else *dst = __builtin_fmaf(skip, xv, o);
-            }
+            if (sub == 0) osm[tt * COLS + lcol] = MODE == 2 ? o : __builtin_fmaf(skip, xv, o);
         };
         float cq[DKQ], ck[DKQ], cw[DKQ], cv, cs, nq[DKQ], nk[DKQ], nw[DKQ], nv, ns;
         read_token(0, cq, ck, cw, cv, cs);
@@ -335,6 +332,16 @@ __global__ __launch_bounds__(256) void gated_linear_scan_kernel(ScanArgs p) {
             token(tt + 1, nq, nk, nw, nv, ns);
         }
         if (tt < nt) token(tt, cq, ck, cw, cv, cs);
+        // the stage's outputs leave together, a token's columns side by side (MODE 2 adds to what MODE 1 wrote)
+        __syncthreads();
+        for (int i = threadIdx.x; i < nt * COLS; i += 256) {
+            const int ot = i / COLS, oc = i - ot * COLS;
+            if (col0 + oc < dv) {
+                float* dst = p.out + (int64_t)(t0 + ot) * p.H * dv + head * dv + col0 + oc;
+                if constexpr (MODE == 2) *dst += osm[i];
+                else *dst = osm[i];
+            }
+        }
     }
     if constexpr (MODE == 2) {
         if (seg != nseg - 1) return;
@@ -443,7 +450,7 @@ void launch_scan_as(const ScanArgs& p, int64_t batch, hipStream_t st) {
     constexpr int CH = (3 * DKQ * SUBS + COLS + 4 + 255) / 256;
     constexpr int TOK = (32 / CH) < 2 ? 2 : (32 / CH);
     const unsigned colblocks = (unsigned)nvh_cdiv(p.dv, COLS);
-    const size_t lds = sizeof(float) * (size_t)TOK * ((3 * p.dk + COLS + 4) & ~3);
+    const size_t lds = sizeof(float) * (size_t)TOK * (((3 * p.dk + COLS + 4) & ~3) + COLS);
     if constexpr (EXACT) {
         if (p.nseg > 1) {
             const dim3 grid((unsigned)batch, (unsigned)p.H, colblocks * (unsigned)p.nseg);

@@ -89,20 +89,18 @@ __device__ __forceinline__ void load8(const A* p, int64_t off, int valid, bool v
     }
 }
 
+// One workgroup per token: its four waves take the experts four at a time in turn, every dot product spread over a wave's
+// lanes (a lane takes 8 consecutive elements of every 512) and summed across it; the logits meet in LDS and the first wave picks.
 template <typename A>
 __global__ __launch_bounds__(256) void moe_route_linear_kernel(const A* __restrict__ x, int64_t ldx, const A* __restrict__ w, const A* __restrict__ bias,
                                                                int32_t* __restrict__ ids, float* __restrict__ weights, float* __restrict__ logits_out,
-                                                               int64_t tokens, int experts, int K, int top, int vec) {
-    const int64_t t = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (t >= tokens) return;
-    const int lane = threadIdx.x & 63;
+                                                               int experts, int K, int top, int vec) {
+    __shared__ float zs[64 * ROUTE_MAX_PER_LANE];
+    const int64_t t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const A* xr = x + t * ldx;
-    float z[ROUTE_MAX_PER_LANE];
-#pragma unroll
-    for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) z[j] = -INFINITY;
-    // eight experts at a time: their loads do not wait for one another; a lane takes 8 consecutive elements of every 512
-    constexpr int EG = 8;
-    for (int e0 = 0; e0 < experts; e0 += EG) {
+    constexpr int EG = 4;
+    for (int e0 = wave * EG; e0 < experts; e0 += 4 * EG) {
         float acc[EG];
 #pragma unroll
         for (int g = 0; g < EG; ++g) acc[g] = 0.f;
@@ -120,14 +118,18 @@ __global__ __launch_bounds__(256) void moe_route_linear_kernel(const A* __restri
 #pragma unroll
         for (int g = 0; g < EG; ++g) {
             const int e = e0 + g;
-            if (e >= experts) break;
-            const float s = wave_sum(acc[g]) + (bias ? (float)bias[e] : 0.f);
-            if (logits_out && lane == 0) logits_out[t * experts + e] = s;
-#pragma unroll
-            for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j)
-                if (lane + 64 * j == e) z[j] = s;
+            const float s = wave_sum(acc[g]) + (bias && e < experts ? (float)bias[e] : 0.f);
+            if (lane == 0 && e < experts) {
+                zs[e] = s;
+                if (logits_out) logits_out[t * experts + e] = s;
+            }
         }
     }
+    __syncthreads();
+    if (wave != 0) return;
+    float z[ROUTE_MAX_PER_LANE];
+#pragma unroll
+    for (int j = 0; j < ROUTE_MAX_PER_LANE; ++j) z[j] = lane + 64 * j < experts ? zs[lane + 64 * j] : -INFINITY;
     float first = 0.f, denom = 0.f;
     for (int r = 0; r < top; ++r) {
         float bv = -INFINITY;
@@ -277,11 +279,11 @@ extern "C" int32_t nvh_moe_route_linear(const void* x, int64_t x_row_stride, con
     NVH_REQUIRE(num_tokens >= 0 && experts > 0 && top > 0 && top <= experts && K > 0 && K < (1 << 30) && x_row_stride >= K, NVH_EINVAL, "nvh_moe_route_linear: bad sizes");
     NVH_REQUIRE(experts <= 64 * ROUTE_MAX_PER_LANE, NVH_ENOSYS, "nvh_moe_route_linear: %ld experts above %d", (long)experts, 64 * ROUTE_MAX_PER_LANE);
     if (num_tokens == 0) return NVH_OK;
-    const dim3 grid((unsigned)nvh_cdiv(num_tokens, 4));
+    const dim3 grid((unsigned)num_tokens);
     hipStream_t st = (hipStream_t)stream;
     const int vec = K % 8 == 0 && x_row_stride % 8 == 0 && nvh_aligned16(x) && nvh_aligned16(w);
-    if (act_f32) moe_route_linear_kernel<float><<<grid, 256, 0, st>>>((const float*)x, x_row_stride, (const float*)w, (const float*)bias, ids, weights, logits_out, num_tokens, (int)experts, (int)K, (int)top, vec);
-    else moe_route_linear_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, x_row_stride, (const bf16*)w, (const bf16*)bias, ids, weights, logits_out, num_tokens, (int)experts, (int)K, (int)top, vec);
+    if (act_f32) moe_route_linear_kernel<float><<<grid, 256, 0, st>>>((const float*)x, x_row_stride, (const float*)w, (const float*)bias, ids, weights, logits_out, (int)experts, (int)K, (int)top, vec);
+    else moe_route_linear_kernel<bf16><<<grid, 256, 0, st>>>((const bf16*)x, x_row_stride, (const bf16*)w, (const bf16*)bias, ids, weights, logits_out, (int)experts, (int)K, (int)top, vec);
     NVH_CHECK_LAUNCH("nvh_moe_route_linear");
     return NVH_OK;
 }
