@@ -38,15 +38,16 @@ __device__ __forceinline__ void gemm_any_bf16_tile(const bf16* __restrict__ x, i
         for (int j = 0; j < 2; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int lr = tid >> 2, lc = (tid & 3) * 16;            // this thread's row and first column of the 64 x 64 tile
     const int64_t xrow = lr < rm.rows ? rm.src(lr) : 0;
-    for (int k0 = 0; k0 < K; k0 += GK) {
-        // stage both tiles
+    // This thread's four 16-byte pieces of the next k-step's tiles (x: 0, 1; w: 2, 3) are loaded while the current step's
+    // products run: a step does not wait for its own loads.
+    bf16x8 pre[4];
+    auto gload = [&](int k0) {
 #pragma unroll
         for (int which = 0; which < 2; ++which) {
             const bf16* src = which ? w : x;
             const int64_t ld = which ? ldw : ldx;
             const int64_t row = which ? n0 + lr : xrow;
             const bool row_ok = which ? n0 + lr < N : lr < rm.rows;
-            bf16* dst = (which ? ws : xs) + lr * GLD + lc;
 #pragma unroll
             for (int half = 0; half < 2; ++half) {
                 const int kc = k0 + lc + half * 8;
@@ -57,10 +58,18 @@ __device__ __forceinline__ void gemm_any_bf16_tile(const bf16* __restrict__ x, i
 #pragma unroll
                     for (int e = 0; e < 8; ++e) v[e] = (row_ok && kc + e < K) ? src[row * ld + kc + e] : (bf16)0.f;
                 }
-                *reinterpret_cast<bf16x8*>(dst + half * 8) = v;
+                pre[which * 2 + half] = v;
             }
         }
+    };
+    gload(0);
+    for (int k0 = 0; k0 < K; k0 += GK) {
+#pragma unroll
+        for (int which = 0; which < 2; ++which)
+#pragma unroll
+            for (int half = 0; half < 2; ++half) *reinterpret_cast<bf16x8*>((which ? ws : xs) + lr * GLD + lc + half * 8) = pre[which * 2 + half];
         __syncthreads();
+        if (k0 + GK < K) gload(k0 + GK);
 #pragma unroll
         for (int ks = 0; ks < GK / 32; ++ks) {
             bf16x8 wf[2], xf[2];
