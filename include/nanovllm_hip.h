@@ -583,7 +583,7 @@ int32_t nvh_logits_scale(const void* logits, int64_t row_stride, float* out, int
  *   S <- diag(w) S + (c k) v^T,  o = S^T q + d v.
  * nvh_gated_linear_scan: operands fp32; q, k [T, qk_groups, dk] (head h reads group h / (H / qk_groups)), w [T, H, dk] or
  * [T, H] (w_scalar), kscale = c [T, H] (NULL: 1), v [T, H, dv], skip = d [H] (NULL: 0); strides are per token.  Sequences,
- * slots and the fresh start as in nvh_delta_scan; out fp32 [T, H dv].  dk <= 256.  segments > 1 (key sizes for which
+ * slots and the fresh start as in nvh_delta_scan; out fp32 [T, H dv].  dk <= 512.  segments > 1 (key sizes for which
  * nvh_scan_segmentable holds; ignored otherwise): a sequence that brings at least segment_min_tokens tokens is cut into that
  * many segments walked side by side and joined in a second launch; ws_states fp32 [batch, H, segments, dv, dk] and ws_decays
  * fp32 [batch, H, segments, dk] are scratch.  Results then differ from the unsegmented form within rounding.

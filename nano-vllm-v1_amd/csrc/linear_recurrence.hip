@@ -551,7 +551,7 @@ extern "C" int32_t nvh_gated_linear_scan(const float* q, int64_t q_stride, const
                                          int64_t segments, int64_t segment_min_tokens, float* ws_states, float* ws_decays, nvh_stream_t stream) {
     NVH_REQUIRE(q && k && w && v && state && slots && context_lens && out, NVH_EINVAL, "nvh_gated_linear_scan: null pointer");
     NVH_REQUIRE(batch >= 0 && heads > 0 && dk > 0 && dv > 0 && qk_groups > 0 && heads % qk_groups == 0, NVH_EINVAL, "nvh_gated_linear_scan: bad sizes");
-    NVH_REQUIRE(dk <= 256, NVH_ENOSYS, "nvh_gated_linear_scan: key size %ld above 256", (long)dk);
+    NVH_REQUIRE(dk <= 512, NVH_ENOSYS, "nvh_gated_linear_scan: key size %ld above 512", (long)dk);
     if (batch == 0) return NVH_OK;
     ScanArgs p{q, k, q_stride, k_stride, (int)qk_groups, w, w_stride, w_scalar, kscale, kscale_stride, v, v_stride, skip, state, slots,
                      cu_seqlens_q, context_lens, out, (int)heads, (int)dk, (int)dv, 1, 1 << 30, ws_states, ws_decays};
@@ -573,14 +573,16 @@ extern "C" int32_t nvh_gated_linear_scan(const float* q, int64_t q_stride, const
             case 16: launch_scan_as<16, 16, true>(p, batch, st); break;
             default:
                 if (dk / 16 <= 8) launch_scan_as<8, 16, false>(p, batch, st);
-                else launch_scan_as<16, 16, false>(p, batch, st);
+                else if (dk / 16 <= 16) launch_scan_as<16, 16, false>(p, batch, st);
+                else launch_scan_as<32, 16, false>(p, batch, st);
         }
     } else {
         const int dkq = (int)(dk + 3) / 4;
         if (dkq <= 8) launch_scan_as<8, 4, false>(p, batch, st);
         else if (dkq <= 16) launch_scan_as<16, 4, false>(p, batch, st);
         else if (dkq <= 32) launch_scan_as<32, 4, false>(p, batch, st);
-        else launch_scan_as<64, 4, false>(p, batch, st);
+        else if (dkq <= 64) launch_scan_as<64, 4, false>(p, batch, st);
+        else launch_scan_as<32, 16, false>(p, batch, st);
     }
     NVH_CHECK_LAUNCH("nvh_gated_linear_scan");
     return NVH_OK;

@@ -254,7 +254,7 @@ def test_scan_against_the_recurrence_written_out():
     from nanovllm import ops
     g = torch.Generator().manual_seed(0)
     for H, G, dk, dv, scalar, lens in [(4, 2, 20, 12, True, [9, 5]), (2, 2, 16, 48, False, [9, 5]), (3, 1, 64, 70, True, [9, 5]), (2, 2, 37, 5, False, [9, 5]),
-                                       (1, 1, 128, 64, False, [9, 5]),
+                                       (1, 1, 128, 64, False, [9, 5]), (1, 1, 300, 6, False, [9, 5]), (1, 1, 512, 20, True, [9, 5]),
                                        # long portions: walked in segments that are joined afterwards (beside a short one that is not)
                                        (2, 1, 32, 24, True, [300, 7]), (1, 1, 64, 16, False, [1, 555]), (2, 2, 16, 8, False, [256, 257])]:
         past = [4, 0]
