@@ -428,6 +428,9 @@ class ModelRunner:
         cfg, hf = self.config, self.config.hf_config
         if self.generic:
             slots = cfg.num_state_slots if cfg.recurrent_state else 0
+            if cfg.num_kvcache_blocks <= 0 and self.generic_block_bytes() == 0:
+                # no layer keeps pages (recurrent mixers only): pages then merely count tokens; enough for every sequence at full length
+                cfg.num_kvcache_blocks = cfg.max_num_seqs * -(-cfg.max_model_len // self.block_size)
             if cfg.num_kvcache_blocks <= 0:
                 free, total = torch.cuda.mem_get_info()
                 stats = torch.cuda.memory_stats()

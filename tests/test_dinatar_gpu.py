@@ -651,6 +651,27 @@ def test_greedy_generation_through_the_engine(loop_case):
         assert out["token_ids"] == toks[len(prompt):]
 
 
+def test_pool_sized_by_the_engine_with_and_without_attention_layers(tmp_path, loop_case):
+    """No page count given: the engine sizes the pool from free memory less the state pools; a model of recurrent mixers only
+    keeps no pages at all and gets a count that merely bounds the tokens."""
+    from nanovllm import LLM, SamplingParams
+    cfg = config([GLA_A, HGRN_B], width=64, vocab=40)
+    recurrent_only = Case(tmp_path, cfg, seed=8)
+    for case, c in ((recurrent_only, cfg), (loop_case, CFG_LOOP)):
+        prompt = tokens_of(c, 9, 3)
+        llm = LLM(case.path, dtype="float32", max_num_seqs=3, max_num_batched_tokens=64, max_model_len=300, gpu_memory_utilization=0.2)
+        try:
+            pages = llm.model_runner.config.num_kvcache_blocks
+            assert pages == 3 * 2 if case is recurrent_only else pages > 100
+            out = llm.generate([prompt], SamplingParams(temperature=0.0, max_tokens=4, ignore_eos=True), use_tqdm=False)[0]
+        finally:
+            llm.exit()
+        toks = list(prompt)
+        for _ in range(4):
+            toks.append(int(R.forward(case.W, c, toks)[-1].argmax()))
+        assert out["token_ids"] == toks[len(prompt):]
+
+
 def test_captured_decode_steps_match_eager_ones(loop_case):
     """One-token steps replayed from the captured graph (routing, expert tiles and states inside it) against the same steps
     run eagerly: several replays, with eager work between them."""
