@@ -148,6 +148,28 @@ __device__ __forceinline__ bf16x8 qknorm_rope_head(bf16x8 x, bf16x8 w, const flo
     return qknorm_rope_head_cs(x, w, c0, c1, s0, s1, c, eps);
 }
 
+// Eight consecutive elements p[off .. off + 7] as floats; those at or beyond `valid` read as zero.  `vec`: 16-byte accesses are allowed.
+template <typename A>
+__device__ __forceinline__ void nvh_load8(const A* p, int64_t off, int valid, bool vec, float (&out)[8]) {
+    if (vec && valid >= 8) {
+        if constexpr (sizeof(A) == 2) {
+            const bf16x8 v = *reinterpret_cast<const bf16x8*>(p + off);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) out[i] = (float)v[i];
+        } else {
+            const f32x4 a = *reinterpret_cast<const f32x4*>(p + off), b = *reinterpret_cast<const f32x4*>(p + off + 4);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                out[i] = a[i];
+                out[4 + i] = b[i];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = i < valid ? (float)p[off + i] : 0.f;
+    }
+}
+
 // ---- sampling pieces shared by the sampler kernels and the LM-head GEMM epilogue ------------------
 struct ValIdx {
     float v;

@@ -128,6 +128,66 @@ __global__ __launch_bounds__(256) void ssd_conv_prep_kernel(SsdPrepArgs p) {
     }
 }
 
+// The same with eight consecutive channels per lane and 16-byte accesses (TAPS known at compile time; channel counts of x, B, C
+// multiples of 8, rows 16-byte aligned): a tap is one load of the inputs and one of the weights instead of eight of each.
+template <typename A, int TAPS>
+__global__ __launch_bounds__(256) void ssd_conv_prep_vec_kernel(SsdPrepArgs p) {
+    const int64_t t = blockIdx.x;
+    const int seq = seq_of_token(p.cu_seqlens_q, p.batch, t);
+    const int lo = p.cu_seqlens_q ? p.cu_seqlens_q[seq] : seq, hi = p.cu_seqlens_q ? p.cu_seqlens_q[seq + 1] : seq + 1;
+    const int j = (int)t - lo;
+    const int slot = p.slots[seq];
+    const bool carried = slot >= 0 && p.context_lens[seq] != hi - lo;
+    const int C = p.inner + 2 * p.gn;
+    const float* st = carried ? p.conv_state + (int64_t)slot * (TAPS - 1) * C : nullptr;
+    for (int c = (blockIdx.y * 256 + threadIdx.x) * 8; c < C; c += 256 * 8 * gridDim.y) {
+        float acc[8], wf[8 * TAPS];                          // wf[i * TAPS + k]: channel c + i, tap k (as the weights lie)
+        if (p.conv_b) {
+            nvh_load8((const A*)p.conv_b, c, 8, true, acc);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = 0.f;
+        }
+#pragma unroll
+        for (int k = 0; k < TAPS; ++k) {
+            float piece[8];
+            nvh_load8((const A*)p.conv_w, (int64_t)c * TAPS + 8 * k, 8, true, piece);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) wf[8 * k + i] = piece[i];
+        }
+#pragma unroll
+        for (int k = 0; k < TAPS; ++k) {                     // tap k multiplies the input TAPS - 1 - k tokens back
+            const int back = TAPS - 1 - k, src = j - back;
+            float in[8];
+            if (src >= 0) {
+                nvh_load8((const A*)p.xbc, (t - back) * p.xbc_stride + c, 8, true, in);
+            } else if (st) {
+                nvh_load8(st, (int64_t)(TAPS - 1 + src) * C + c, 8, true, in);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) in[i] = 0.f;
+            }
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = __builtin_fmaf(wf[i * TAPS + k], in[i], acc[i]);
+        }
+        float* dst = c < p.inner ? p.ov + t * p.inner + c : (c < p.inner + p.gn ? p.ok + t * p.gn + (c - p.inner) : p.oq + t * p.gn + (c - p.inner - p.gn));
+        f32x4 lo4, hi4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            lo4[i] = silu_(acc[i]);
+            hi4[i] = silu_(acc[4 + i]);
+        }
+        *reinterpret_cast<f32x4*>(dst) = lo4;
+        *reinterpret_cast<f32x4*>(dst + 4) = hi4;
+    }
+    if (blockIdx.y != 0) return;
+    for (int h = threadIdx.x; h < p.H; h += 256) {
+        const float dt = softplus_(ldf((const A*)p.dt, t * p.dt_stride + h) + ldf((const A*)p.dt_bias, h));
+        p.oc[t * p.H + h] = dt;
+        p.ow[t * p.H + h] = expf(-expf(ldf((const A*)p.a_log, h)) * dt);
+    }
+}
+
 // One thread per (sequence, channel): slot s of the new state is input number n + s - (taps - 1) of [carried | this step's].
 // Ascending s only ever reads carried entries at or above the one it writes.
 template <typename A>
@@ -516,9 +576,24 @@ extern "C" int32_t nvh_ssd_conv_prep(const void* xbc, int64_t xbc_stride, const 
     p.ov = out_x, p.ok = out_b, p.oq = out_c, p.oc = out_dt, p.ow = out_decay;
     hipStream_t st = (hipStream_t)stream;
     // few tokens: the channels are spread over more workgroups (a token's row is short work for one)
-    const dim3 grid((unsigned)num_tokens, (unsigned)(num_tokens >= 512 ? 1 : std::min<int64_t>(nvh_cdiv(inner + 2 * gn, 256), 16)));
-    if (act_f32) ssd_conv_prep_kernel<float><<<grid, 256, 0, st>>>(p);
-    else ssd_conv_prep_kernel<bf16><<<grid, 256, 0, st>>>(p);
+    const int64_t esz = act_f32 ? 4 : 2, per_lane = 16 / esz;            // elements per 16 bytes
+    const bool vec = taps >= 2 && taps <= 4 && inner % 8 == 0 && gn % 8 == 0 && xbc_stride % per_lane == 0 && nvh_aligned16(xbc) && nvh_aligned16(conv_w) &&
+                     (!conv_b || nvh_aligned16(conv_b)) && nvh_aligned16(conv_state) && nvh_aligned16(out_x) && nvh_aligned16(out_b) && nvh_aligned16(out_c);
+    const int64_t lanes = vec ? (inner + 2 * gn) / 8 : inner + 2 * gn;
+    const dim3 grid((unsigned)num_tokens, (unsigned)(num_tokens >= 512 ? 1 : std::min<int64_t>(nvh_cdiv(lanes, 256), 16)));
+    if (vec) {
+#define NVH_CONV_VEC(TAPS)                                                        \
+    if (act_f32) ssd_conv_prep_vec_kernel<float, TAPS><<<grid, 256, 0, st>>>(p); \
+    else ssd_conv_prep_vec_kernel<bf16, TAPS><<<grid, 256, 0, st>>>(p)
+        if (taps == 2) { NVH_CONV_VEC(2); }
+        else if (taps == 3) { NVH_CONV_VEC(3); }
+        else { NVH_CONV_VEC(4); }
+#undef NVH_CONV_VEC
+    } else if (act_f32) {
+        ssd_conv_prep_kernel<float><<<grid, 256, 0, st>>>(p);
+    } else {
+        ssd_conv_prep_kernel<bf16><<<grid, 256, 0, st>>>(p);
+    }
     NVH_CHECK_LAUNCH("nvh_ssd_conv_prep");
     return NVH_OK;
 }

@@ -67,28 +67,6 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const float* __restrict_
 
 // The same with the router's product inside: z[e] = x . w[e] + bias[e] in fp32, every expert's dot product spread over the
 // wave's lanes (lane l takes elements l, l + 64, ... of the row) and summed across it.
-// Eight consecutive elements p[off .. off + 7] as floats; those at or beyond `valid` read as zero.  `vec`: 16-byte accesses are allowed.
-template <typename A>
-__device__ __forceinline__ void load8(const A* p, int64_t off, int valid, bool vec, float (&out)[8]) {
-    if (vec && valid >= 8) {
-        if constexpr (sizeof(A) == 2) {
-            const bf16x8 v = *reinterpret_cast<const bf16x8*>(p + off);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) out[i] = (float)v[i];
-        } else {
-            const f32x4 a = *reinterpret_cast<const f32x4*>(p + off), b = *reinterpret_cast<const f32x4*>(p + off + 4);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                out[i] = a[i];
-                out[4 + i] = b[i];
-            }
-        }
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) out[i] = i < valid ? (float)p[off + i] : 0.f;
-    }
-}
-
 // One workgroup per token: its four waves take the experts four at a time in turn, every dot product spread over a wave's
 // lanes (a lane takes 8 consecutive elements of every 512) and summed across it; the logits meet in LDS and the first wave picks.
 template <typename A>
@@ -106,11 +84,11 @@ __global__ __launch_bounds__(256) void moe_route_linear_kernel(const A* __restri
         for (int g = 0; g < EG; ++g) acc[g] = 0.f;
         for (int k0 = lane * 8; k0 < K; k0 += 512) {
             float xv[8];
-            load8(xr, k0, K - k0, vec, xv);
+            nvh_load8(xr, k0, K - k0, vec, xv);
 #pragma unroll
             for (int g = 0; g < EG; ++g) {
                 float wv[8];
-                load8(w + (int64_t)min(e0 + g, experts - 1) * K, k0, K - k0, vec, wv);
+                nvh_load8(w + (int64_t)min(e0 + g, experts - 1) * K, k0, K - k0, vec, wv);
 #pragma unroll
                 for (int i = 0; i < 8; ++i) acc[g] = __builtin_fmaf(xv[i], wv[i], acc[g]);
             }

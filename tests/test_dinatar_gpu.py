@@ -30,6 +30,13 @@ PAR_A = {"type": "parallel", "mlp": DENSE,
 PAR_B = {"type": "parallel", "mlp": MOE_A,
          "mixer": {"left": {"heads": 4, "kv_heads": 4, "dim": 16, "vdim": 16, "scale": 0.25, "mask": {"size": 70, "keep_first": 0}},
                    "right": {"heads": 6, "vdim": 16, "state": 16, "groups": 1, "conv": 4, "norm_groups": 3}}}
+# right: channel counts and a projection row that are multiples of 8 (the convolution's 16-byte form), three taps / two taps
+PAR_C = {"type": "parallel", "mlp": None,
+         "mixer": {"left": {"heads": 2, "kv_heads": 1, "dim": 8, "vdim": 8, "scale": 0.35, "mask": {"size": 40, "keep_first": 1}},
+                   "right": {"heads": 8, "vdim": 8, "state": 8, "groups": 2, "conv": 3, "norm_groups": 2}}}
+PAR_D = {"type": "parallel", "mlp": DENSE,
+         "mixer": {"left": {"heads": 2, "kv_heads": 2, "dim": 8, "vdim": 24, "scale": 0.35, "mask": {"size": 9, "keep_first": 2}},
+                   "right": {"heads": 16, "vdim": 4, "state": 24, "groups": 1, "conv": 2, "norm_groups": 1}}}
 HGRN_A = {"type": "hgrn2", "mixer": {"heads": 3, "dim": 20, "vdim": 28}, "mlp": MOE_B}
 HGRN_B = {"type": "hgrn2", "mixer": {"heads": 2, "dim": 32, "vdim": 16}, "mlp": None}
 GLA_A = {"type": "gla", "mixer": {"heads": 2, "dim": 16, "vdim": 48, "tau": 8.0}, "mlp": DENSE}
@@ -210,8 +217,9 @@ def run_schedule(rp, case, requests: dict, schedule: list, dtype: str, tol=None)
 
 
 # ----------------------------------------------------------------------------------------------------- single mechanisms
-@pytest.mark.parametrize("layer", [PAR_A, PAR_B, HGRN_A, HGRN_B, GLA_A, GLA_B],
-                         ids=["parallel(gqa, ragged sizes)+dense", "parallel(heads of 16)+moe", "hgrn2+moe(top 1)", "hgrn2", "gla+dense", "gla+moe"])
+@pytest.mark.parametrize("layer", [PAR_A, PAR_B, PAR_C, PAR_D, HGRN_A, HGRN_B, GLA_A, GLA_B],
+                         ids=["parallel(gqa, ragged sizes)+dense", "parallel(heads of 16)+moe", "parallel(3 taps, aligned)", "parallel(2 taps, aligned)+dense",
+                              "hgrn2+moe(top 1)", "hgrn2", "gla+dense", "gla+moe"])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_one_layer_stream_matches(tmp_path, layer, dtype):
     """One layer of each kind, no loop: the residual stream after it and the logits."""
@@ -399,10 +407,10 @@ def test_portions_of_every_size_give_the_same_logits(loop_case):
 def test_cutting_does_not_change_a_bit_of_the_recurrent_path(tmp_path):
     """Recurrent mixers only (no attention, whose key tiles see the cut): one piece, portions and single tokens give
     identical logits, the convolution's carried inputs included."""
-    mamba_only = copy.deepcopy(PAR_A)
-    cfg = config([HGRN_B, GLA_A, mamba_only], width=64, vocab=64)
+    cfg = config([HGRN_B, GLA_A, copy.deepcopy(PAR_A), copy.deepcopy(PAR_C)], width=64, vocab=64)
     w = random_weights(cfg, 5)
-    w["l2.mix.left.out"] = torch.zeros_like(w["l2.mix.left.out"])
+    w["l2.mix.left.out"] = torch.zeros_like(w["l2.mix.left.out"])            # the attention branches are switched off
+    w["l3.mix.left.out"] = torch.zeros_like(w["l3.mix.left.out"])
     case = Case(tmp_path, cfg, weights=w)
     toks = tokens_of(cfg, 48, 2)
     rp = case.replay("float32")
